@@ -1,0 +1,186 @@
+/*
+ * tensorlib_amd.h : C ABI of the MI355X (gfx950) device backend for tensorLib's
+ * matrix-multiplication hot path.
+ *
+ * Every entry point is what a `Device<dtype>` subclass of the reference
+ * (tensorLib/include/device/Device.hpp:5-110) forwards to: plain device pointers and
+ * sizes, no C++ types, no exceptions across the boundary.  "f16" buffers hold IEEE
+ * binary16 values (the reference's `half`); element counts are in elements, not bytes.
+ *
+ * Conventions
+ *   - Return value: 0 on success, a negative TL_E* code otherwise; tl_last_error()
+ *     returns the message of the calling thread's last failure.
+ *   - All pointers named A/B/C/x/W/y/in/out/src/dst are DEVICE pointers unless the
+ *     parameter is called host_*.
+ *   - Work is enqueued on one in-order HIP stream (the null stream unless
+ *     tl_set_stream() was called) and is asynchronous w.r.t. the host, like the
+ *     reference's default-stream launches (tensorLib/src/device/cuda/CUDA.cu).
+ *   - Matrices are dense row-major.  The matmul operand contract is the reference's:
+ *     A[M,K], B[N,K] ("col-major B"), C[M,N] (tensorLib/src/ops/matmul.cpp:265-268).
+ */
+#ifndef TENSORLIB_AMD_H
+#define TENSORLIB_AMD_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define TL_OK 0
+#define TL_EINVAL (-1)   /* bad argument (null pointer, misaligned, size out of range) */
+#define TL_EHIP (-2)     /* a HIP runtime call failed */
+#define TL_ENOMEM (-3)   /* device allocation failed */
+#define TL_ELIMIT (-4)   /* size exceeds a documented limit of the entry point */
+
+/* ---------------------------------------------------------------- runtime ---- */
+
+/* Select the GPU, read its properties, create library state.  Idempotent.
+ * Replaces the implicit CUDA context creation of the first cudaMalloc
+ * (tensorLib/src/device/cuda/CUDA.cu:16-19). */
+int tl_init(int device_ordinal);
+
+/* Message of the calling thread's last failing tl_* call ("" if none).
+ * Replaces the print-and-exit of CUDA_CHECK (tensorLib/include/device/cuda/CUDA.cuh:131-151). */
+const char* tl_last_error(void);
+
+/* Library version string, e.g. "tensorlib_amd 0.1 gfx950". */
+const char* tl_version(void);
+
+/* Number of compute units and wavefront size of the selected GPU (0 before tl_init). */
+int tl_device_cu_count(void);
+
+/* Enqueue all later work on `hip_stream` (a hipStream_t; NULL = null stream).
+ * The reference uses the default stream everywhere (tensorLib/src/device/cuda/gemm.cu). */
+int tl_set_stream(void* hip_stream);
+void* tl_get_stream(void);
+
+/* Device memory: CUDA<dtype>::CUDA(size) / ~CUDA() (tensorLib/src/device/cuda/CUDA.cu:16-32). */
+int tl_malloc(void** dev_ptr, size_t bytes);
+int tl_free(void* dev_ptr);
+
+/* Copies.  h2d/d2h synchronise with the stream before returning, like the 1-element
+ * cudaMemcpy of getDataLinear/setDataLinear (tensorLib/src/device/cuda/CUDA.cu:71-81)
+ * and the weight loader's cudaMemcpy (model/llama2_7b/src/main.cpp:53-57). */
+int tl_memcpy_h2d(void* dst, const void* host_src, size_t bytes);
+int tl_memcpy_d2h(void* host_dst, const void* src, size_t bytes);
+int tl_memcpy_d2d(void* dst, const void* src, size_t bytes);
+int tl_synchronize(void);
+
+/* ------------------------------------------------------- the hot path ---- */
+
+/* C[M,N] = A[M,K] . B[N,K]^T, fp32 accumulation, one rounding to fp16 at the end.
+ * Replaces Device<half>::matmul2d (tensorLib/include/device/Device.hpp:22) as
+ * implemented by CUDA<half>::matmul2d (tensorLib/src/device/cuda/gemm.cu:153-172);
+ * numerics follow CPU<half>::matmul2d (tensorLib/src/device/cpu/CPU.cpp:76-89).
+ * M == 1 takes the GEMV path, M > 1 the MFMA GEMM path; any M,N,K >= 1 is accepted
+ * (unaligned shapes take a slower generic kernel).  C must not alias A or B. */
+int tl_matmul2d_f16(const void* A, const void* B, void* C, size_t M, size_t N, size_t K);
+
+/* y[N] = W[N,K] . x[K].  Replaces gemv_v6 / gemv_v4
+ * (tensorLib/src/device/cuda/gemv.cu:379-450, :260-300).  Fast path needs K % 8 == 0
+ * and 16-byte aligned x and W; otherwise a scalar-load kernel runs. */
+int tl_gemv_f16(const void* x, const void* W, void* y, size_t N, size_t K);
+
+/* C[M,N] = A[M,K] . B[N,K]^T on the matrix cores.  Replaces hgemm_cublas
+ * (tensorLib/src/device/cuda/hgemm.cu:20-38) but keeps fp32 accumulation, which the
+ * cuBLAS call with fp16 alpha/beta does not guarantee. */
+int tl_hgemm_f16(const void* A, const void* B, void* C, size_t M, size_t N, size_t K);
+
+/* Batched form of the loop in ops::matmul<dtype>::call2
+ * (tensorLib/src/ops/matmul.cpp:297-321): for b in [0,batch):
+ *   C + b*strideC = matmul2d(A + b*strideA, B + b*strideB), strides in elements
+ * (0 = operand broadcast over the batch).  One launch instead of `batch` launches. */
+int tl_matmul2d_batched_f16(const void* A, const void* B, void* C, size_t M, size_t N, size_t K,
+                            size_t batch, size_t strideA, size_t strideB, size_t strideC);
+
+/* fp32 / int32 matmul2d for Device<float> / Device<int> (same operand contract;
+ * tensorLib/src/device/cpu/CPU.cpp:76-89 with dtype=float/int: fp32 accumulate then
+ * cast).  Plain tiled kernels; not part of the fp16 hot path. */
+int tl_matmul2d_f32(const void* A, const void* B, void* C, size_t M, size_t N, size_t K);
+
+/* Force a kernel variant for benchmarking/tests: 0 = automatic dispatch.  The variant
+ * names are listed by tl_gemv_variant_name()/tl_hgemm_variant_name() (NULL past the end). */
+int tl_set_gemv_variant(int variant);
+int tl_set_hgemm_variant(int variant);
+const char* tl_gemv_variant_name(int variant);
+const char* tl_hgemm_variant_name(int variant);
+/* Tuning hook: cap the GEMV grid at `waves` resident wavefronts per compute unit (0 = default). */
+int tl_set_gemv_grid_waves_per_cu(int waves);
+
+/* ------------------------------- small kernels that keep decode on the GPU ---- */
+
+/* out[t,:] = in[t,:] * weight[:] / sqrt(mean(in[t,:]^2) + eps), fp32 math, one rounding.
+ * Replaces CUDA<dtype>::rms_norm (tensorLib/include/device/cuda/CUDA.cuh:108,
+ * tensorLib/src/device/cuda/rms_norm.cu:139-184), called from
+ * nn::RMSNorm::forward_fused_cuda (tensorLib/src/nn/rmsNorm.cpp:62-94). */
+int tl_rms_norm_f16(void* out, const void* in, const void* weight, float eps,
+                    int hidden_size, int num_tokens);
+
+/* Interleaved-pair rotary embedding on a contiguous [B,T,n_heads,head_dim] tensor;
+ * in == out is allowed.  Replaces Device::apply_rotary_emb
+ * (tensorLib/include/device/Device.hpp:94-101; tensorLib/src/device/cuda/CUDA.cu:405-437;
+ * numerics per tensorLib/src/device/cpu/CPU.cpp:427-461). */
+int tl_apply_rotary_emb_f16(const void* in, void* out, int start_pos, int B, int T,
+                            int n_heads, int head_dim);
+
+/* Row softmax over the last dimension of a contiguous [rows, cols] matrix; in == out
+ * allowed.  Replaces Device::softmax (Device.hpp:79; tensorLib/src/device/cuda/softmax.cu:21-82;
+ * tensorLib/src/device/cpu/softmax.cpp:9-31).  Max/sum are carried in fp32. */
+int tl_softmax_f16(void* out, const void* in, size_t rows, size_t cols);
+
+/* Elementwise: out = silu(in) = in / (1 + exp(-in)) evaluated in fp32
+ * (tensorLib/src/device/cuda/CUDA.cu:334-347; Device.hpp:57). */
+int tl_silu_f16(void* out, const void* in, size_t n);
+
+/* Elementwise binary ops on halves, one rounding each (Device.hpp:62-65;
+ * tensorLib/include/device/cuda/binary.cuh:3-74).  op: 0 add, 1 sub, 2 mul, 3 div. */
+int tl_binary_f16(void* out, const void* a, const void* b, size_t n, int op);
+/* Same with a scalar right operand given as the 16 bits of a half (Device.hpp:66-70). */
+int tl_binary_scalar_f16(void* out, const void* a, uint16_t scalar_bits, size_t n, int op);
+
+/* out[i] = base[offset + sum_d idx_d(i) * stride[d]] for the row-major index i over
+ * `shape` (Device::contiguous, Device.hpp:30-35; tensorLib/src/device/cuda/CUDA.cu:83-116).
+ * ndim <= 8.  host_shape/host_stride are HOST arrays of ndim ints. */
+int tl_contiguous_f16(void* out, const void* base, const int* host_shape, const int* host_stride,
+                      int ndim, size_t offset, size_t n);
+/* base[offset + sum_d idx_d(i) * stride[d]] = src[i] (Device::setItemEwise,
+ * Device.hpp:36-41; tensorLib/src/device/cuda/CUDA.cu:118-151). */
+int tl_set_item_ewise_f16(void* base, const void* src, const int* host_shape, const int* host_stride,
+                          int ndim, size_t offset, size_t n);
+
+/* out[r] = index of the first maximum of in[r*reduce_size .. +reduce_size)
+ * (Device::argmax, Device.hpp:77; first-max-wins like tensorLib/src/device/cpu/CPU.cpp:356-372). */
+int tl_argmax_f16(int* out, const void* in, size_t reduce_size, size_t num_elements);
+
+/* out[t,:] = table[ids[t],:] for t < n_tokens; ids is a DEVICE int32 array.
+ * Replaces the per-token select+setItem loop of nn::Embedding::forward
+ * (tensorLib/src/nn/embedding.cpp:47-81) without the per-token host read. */
+int tl_embedding_f16(void* out, const void* table, const int* ids, int n_tokens, int dim, int vocab);
+
+/* out[i] = value for i < n (Device::full, Device.hpp:25). */
+int tl_full_f16(void* out, uint16_t value_bits, size_t n);
+
+/* ------------------------------------------ fused forms used by the driver ---- */
+
+/* out = silu(a) * b in fp32, one rounding: FeedForward's silu + EwiseMul
+ * (model/llama2_7b/src/Transformer.cpp:137-141) in one pass. */
+int tl_silu_mul_f16(void* out, const void* a, const void* b, size_t n);
+
+/* Single-token attention over a [max_seq, n_heads, head_dim] KV cache read in place:
+ * out[h,:] = softmax(q[h,:] . K[0:T,h,:]^T / half(sqrt(head_dim))) . V[0:T,h,:].
+ * Replaces the gather + 2*n_heads gemv_v4 launches + scale + softmax of
+ * Attention::forward at seqlen 1 (model/llama2_7b/src/Transformer.cpp:55-109). */
+int tl_decode_attention_f16(void* out, const void* q, const void* cache_k, const void* cache_v,
+                            int T, int n_heads, int head_dim);
+
+/* mask[r,i,j] = (j > start_pos + i) ? -inf : 0 for r < reps, i < seqlen, j < start_pos+seqlen.
+ * Replaces the element-by-element host loop of Transformer::get_mask
+ * (model/llama2_7b/src/Transformer.cpp:231-261). */
+int tl_causal_mask_f16(void* mask, int reps, int seqlen, int start_pos);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TENSORLIB_AMD_H */

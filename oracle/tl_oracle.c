@@ -1,0 +1,387 @@
+/*
+ * tl_oracle.c : CPU restatement of tensorLib's CPU (OpenMP) backend for the matmul hot
+ * path and the small ops around it.  TEST INFRASTRUCTURE ONLY: this file is the checker
+ * the GPU kernels are compared against and the CPU baseline that is timed beside them.
+ * Nothing in the shipped library links, loads or calls it.
+ *
+ * Each function cites the reference lines it restates (paths relative to the reference
+ * tree).  `half` is carried as uint16_t bit patterns; conversions are done in software
+ * (round-to-nearest-even), like the host-side __half2float/__float2half the reference's
+ * CPU backend gets from cuda_fp16.h (tensorLib/include/device/cpu/CPU.hpp:8).
+ *
+ * Parity pins (what each function is checked against, see tests/test_oracle_*.py):
+ *   conversions          : exhaustive against numpy float16 (all 65536 halves; float
+ *                          boundaries, ties, subnormals, overflow)
+ *   tlo_matmul2d_f16     : integer-valued exact cases, identity / unit-vector cases,
+ *                          float64 numpy matmul, pure-Python triple loop on tiny shapes
+ *   tlo_rope_f16         : complex-multiply closed form (tensorLib/test/python/test_ops.py:65-86)
+ *   tlo_softmax_f16_f32  : scipy.special.softmax in float64
+ *   tlo_rms_norm_*       : x * rsqrt(mean(x^2)+eps) * w in float64
+ *   tlo_silu_f16, binary : float64 closed forms
+ *   contiguous/set_item  : numpy as_strided
+ *   argmax               : numpy argmax (first maximum)
+ * PARITY UNPINNED (the reference cannot be compiled in the authoring container: it needs
+ * cuda_fp16.h, and writing a stand-in header is not allowed): the *bit-exact* half-carried
+ * chains tlo_softmax_f16_literal, tlo_rms_norm_f16_plain_literal and
+ * tlo_silu_f16_cpu_literal.  They follow the reference text op by op but no golden vector
+ * exists to confirm the last bit; they are only used to REPORT the distance between the
+ * fp32-accumulating GPU kernels and the literal CPU half chain, never as a gate.
+ */
+#include <math.h>
+#include <stddef.h>
+#include <stdint.h>
+#include <string.h>
+#include <stdlib.h>
+#ifdef _OPENMP
+#include <omp.h>
+#endif
+
+typedef uint16_t h16;
+
+/* ------------------------------------------------------------ conversions ---- */
+
+static float g_h2f[65536];
+static int g_h2f_ready = 0;
+
+static float h2f_slow(h16 h) {
+    uint32_t sign = ((uint32_t)h & 0x8000u) << 16;
+    uint32_t e = (h >> 10) & 0x1fu;
+    uint32_t m = h & 0x3ffu;
+    uint32_t bits;
+    if (e == 0) {
+        if (m == 0) {
+            bits = sign;
+        } else { /* subnormal: m * 2^-24 */
+            int shift = 0;
+            while ((m & 0x400u) == 0) { m <<= 1; shift++; }
+            m &= 0x3ffu;
+            bits = sign | ((uint32_t)(127 - 14 - shift) << 23) | (m << 13);
+        }
+    } else if (e == 31) {
+        bits = sign | 0x7f800000u | (m << 13);
+    } else {
+        bits = sign | ((e + 112u) << 23) | (m << 13);
+    }
+    float f;
+    memcpy(&f, &bits, 4);
+    return f;
+}
+
+__attribute__((constructor)) static void tlo_init_tables(void) {
+    for (uint32_t i = 0; i < 65536; ++i) g_h2f[i] = h2f_slow((h16)i);
+    g_h2f_ready = 1;
+}
+
+static inline float h2f(h16 h) { return g_h2f[h]; }
+
+/* float -> half, round to nearest even, overflow to inf, NaN kept quiet. */
+static inline h16 f2h(float f) {
+    uint32_t x;
+    memcpy(&x, &f, 4);
+    uint32_t sign = (x >> 16) & 0x8000u;
+    x &= 0x7fffffffu;
+    if (x > 0x7f800000u) return (h16)(sign | 0x7e00u | ((x >> 13) & 0x1ffu)); /* NaN */
+    if (x >= 0x477ff000u) return (h16)(sign | 0x7c00u); /* >= 65520 rounds to inf (incl. inf) */
+    if (x < 0x38800000u) { /* below 2^-14: result is a half subnormal (or zero) */
+        /* adding 0.5f aligns the value so that the float adder performs the RNE rounding
+           to a multiple of 2^-24; the low mantissa bits then are the half's bits. */
+        float v, magic = 0.5f;
+        memcpy(&v, &x, 4);
+        v += magic;
+        uint32_t r, mb;
+        memcpy(&r, &v, 4);
+        memcpy(&mb, &magic, 4);
+        return (h16)(sign | (r - mb));
+    }
+    uint32_t odd = (x >> 13) & 1u;
+    x += 0xc8000000u + 0xfffu + odd; /* rebias exponent by (15-127)<<23, round */
+    return (h16)(sign | (x >> 13));
+}
+
+/* exposed for the conversion tests */
+void tlo_h2f(const h16* in, float* out, size_t n) {
+    for (size_t i = 0; i < n; ++i) out[i] = h2f(in[i]);
+}
+void tlo_f2h(const float* in, h16* out, size_t n) {
+    for (size_t i = 0; i < n; ++i) out[i] = f2h(in[i]);
+}
+
+int tlo_max_threads(void) {
+#ifdef _OPENMP
+    return omp_get_max_threads();
+#else
+    return 1;
+#endif
+}
+
+/* ------------------------------------------------------------------ matmul ---- */
+
+/* CPU<half>::matmul2d, tensorLib/src/device/cpu/CPU.cpp:76-89:
+ * omp parallel for collapse(2) over (i,j); float sum over k ascending; one cast. */
+void tlo_matmul2d_f16(const h16* A, const h16* B, h16* C, size_t M, size_t N, size_t K) {
+#pragma omp parallel for collapse(2)
+    for (long i = 0; i < (long)M; i++) {
+        for (long j = 0; j < (long)N; j++) {
+            float sum = 0.0f;
+            for (size_t k = 0; k < K; k++) {
+                sum += h2f(A[i * K + k]) * h2f(B[j * K + k]);
+            }
+            C[i * N + j] = f2h(sum);
+        }
+    }
+}
+
+/* Same arithmetic for a list of (i,j) entries only (sampled parity at sizes where the
+ * full O(MNK) loop is too slow). */
+void tlo_matmul2d_f16_entries(const h16* A, const h16* B, h16* out, const int64_t* ii,
+                              const int64_t* jj, size_t n_entries, size_t K) {
+#pragma omp parallel for
+    for (long e = 0; e < (long)n_entries; e++) {
+        const h16* a = A + (size_t)ii[e] * K;
+        const h16* b = B + (size_t)jj[e] * K;
+        float sum = 0.0f;
+        for (size_t k = 0; k < K; k++) sum += h2f(a[k]) * h2f(b[k]);
+        out[e] = f2h(sum);
+    }
+}
+
+/* CPU<float>::matmul2d, same lines with dtype = float. */
+void tlo_matmul2d_f32(const float* A, const float* B, float* C, size_t M, size_t N, size_t K) {
+#pragma omp parallel for collapse(2)
+    for (long i = 0; i < (long)M; i++) {
+        for (long j = 0; j < (long)N; j++) {
+            float sum = 0.0f;
+            for (size_t k = 0; k < K; k++) sum += A[i * K + k] * B[j * K + k];
+            C[i * N + j] = sum;
+        }
+    }
+}
+
+/* The batch loop of ops::matmul<dtype>::call2, tensorLib/src/ops/matmul.cpp:297-321,
+ * with element strides (0 = broadcast operand). */
+void tlo_matmul2d_batched_f16(const h16* A, const h16* B, h16* C, size_t M, size_t N, size_t K,
+                              size_t batch, size_t sA, size_t sB, size_t sC) {
+    for (size_t b = 0; b < batch; ++b)
+        tlo_matmul2d_f16(A + b * sA, B + b * sB, C + b * sC, M, N, K);
+}
+
+/* ----------------------------------------------------------------- RoPE ---- */
+
+/* CPU<half>::apply_rotary_emb, tensorLib/src/device/cpu/CPU.cpp:427-461.
+ * theta in fp32; cos/sin rounded to half; each half operator rounds (host __half ops). */
+void tlo_rope_f16(const h16* in, h16* out, int start_pos, int B, int T, int n_heads, int head_dim) {
+#pragma omp parallel for collapse(3)
+    for (int b = 0; b < B; b++)
+        for (int t = 0; t < T; t++)
+            for (int h = 0; h < n_heads; h++)
+                for (int d = 0; d < head_dim; d += 2) {
+                    size_t off = (((size_t)b * T + t) * n_heads + h) * head_dim + d;
+                    float theta = (float)(start_pos + t) * 1.0f /
+                                  powf(10000.0f, (float)d / (float)head_dim);
+                    float c = h2f(f2h(cosf(theta)));
+                    float s = h2f(f2h(sinf(theta)));
+                    float v0 = h2f(in[off]), v1 = h2f(in[off + 1]);
+                    float p0 = h2f(f2h(v0 * c)), p1 = h2f(f2h(v1 * s));
+                    float p2 = h2f(f2h(v0 * s)), p3 = h2f(f2h(v1 * c));
+                    h16 re = f2h(p0 - p1), im = f2h(p2 + p3);
+                    out[off] = re;
+                    out[off + 1] = im;
+                }
+}
+
+/* --------------------------------------------------------------- softmax ---- */
+
+/* Softmax with fp32 max/sum and one rounding: the *intended* value of
+ * tensorLib/src/device/cpu/softmax.cpp:9-31 (gate for the GPU kernel). */
+void tlo_softmax_f16_f32(const h16* in, h16* out, size_t rows, size_t cols) {
+#pragma omp parallel for
+    for (long i = 0; i < (long)rows; i++) {
+        const h16* x = in + i * cols;
+        float mx = h2f(x[0]);
+        for (size_t j = 1; j < cols; j++) mx = fmaxf(mx, h2f(x[j]));
+        float sum = 0.0f;
+        for (size_t j = 0; j < cols; j++) sum += expf(h2f(x[j]) - mx);
+        for (size_t j = 0; j < cols; j++) out[i * cols + j] = f2h(expf(h2f(x[j]) - mx) / sum);
+    }
+}
+
+/* Literal half chain of softmaxImpl<half>, tensorLib/src/device/cpu/softmax.cpp:9-31:
+ * half subtraction, exp rounded to half, sum carried in half, half division.
+ * PARITY UNPINNED (see header). */
+void tlo_softmax_f16_literal(const h16* in, h16* out, size_t rows, size_t cols) {
+#pragma omp parallel for
+    for (long i = 0; i < (long)rows; i++) {
+        const h16* x = in + i * cols;
+        h16* o = out + i * cols;
+        float mx = h2f(x[0]);
+        for (size_t j = 1; j < cols; j++)
+            if (h2f(x[j]) > mx) mx = h2f(x[j]);
+        h16 sum = 0;
+        for (size_t j = 0; j < cols; j++) {
+            float d = h2f(f2h(h2f(x[j]) - mx));
+            o[j] = f2h(expf(d));
+            sum = f2h(h2f(sum) + h2f(o[j]));
+        }
+        for (size_t j = 0; j < cols; j++) o[j] = f2h(h2f(o[j]) / h2f(sum));
+    }
+}
+
+/* --------------------------------------------------------------- RMSNorm ---- */
+
+/* rms_norm_kernel_v1, tensorLib/src/device/cuda/rms_norm.cu:139-167: fp32 sum of squares,
+ * rms = half(sqrtf(sum/H + eps)), o = (x*w)/rms with each half operator rounding.
+ * This is what the model executes on the reference's GPU path
+ * (tensorLib/src/nn/rmsNorm.cpp:98-106). */
+void tlo_rms_norm_f16_fused(const h16* in, const h16* w, h16* out, float eps, int hidden, int tokens) {
+#pragma omp parallel for
+    for (int t = 0; t < tokens; t++) {
+        const h16* x = in + (size_t)t * hidden;
+        float sum = 0.0f;
+        for (int i = 0; i < hidden; i++) sum += h2f(x[i]) * h2f(x[i]);
+        float rms = h2f(f2h(sqrtf(sum / (float)hidden + eps)));
+        for (int i = 0; i < hidden; i++) {
+            float xw = h2f(f2h(h2f(x[i]) * h2f(w[i])));
+            out[(size_t)t * hidden + i] = f2h(xw / rms);
+        }
+    }
+}
+
+/* x * rsqrt(mean(x^2)+eps) * w in double, one rounding: the mathematical definition
+ * (script/model.py:33-38) both reference variants approximate. */
+void tlo_rms_norm_f16_exact(const h16* in, const h16* w, h16* out, float eps, int hidden, int tokens) {
+#pragma omp parallel for
+    for (int t = 0; t < tokens; t++) {
+        const h16* x = in + (size_t)t * hidden;
+        double sum = 0.0;
+        for (int i = 0; i < hidden; i++) sum += (double)h2f(x[i]) * (double)h2f(x[i]);
+        double r = 1.0 / sqrt(sum / (double)hidden + (double)eps);
+        for (int i = 0; i < hidden; i++)
+            out[(size_t)t * hidden + i] = f2h((float)((double)h2f(x[i]) * r * (double)h2f(w[i])));
+    }
+}
+
+/* Literal CPU half chain of RMSNorm::forward_plain, tensorLib/src/nn/rmsNorm.cpp:14-56
+ * through CPU<half> ops (pow: CPU.cpp:300-312; mean = sequential half sum then half
+ * divide: CPU.cpp:340-354,389-395; scalar add; rsqrt: CPU.cpp:241-256; two half muls).
+ * PARITY UNPINNED (see header). */
+void tlo_rms_norm_f16_plain_literal(const h16* in, const h16* w, h16* out, float eps, int hidden, int tokens) {
+#pragma omp parallel for
+    for (int t = 0; t < tokens; t++) {
+        const h16* x = in + (size_t)t * hidden;
+        h16 acc = f2h(powf(h2f(x[0]), 2.0f));
+        for (int i = 1; i < hidden; i++) {
+            h16 sq = f2h(powf(h2f(x[i]), 2.0f));
+            acc = f2h(h2f(acc) + h2f(sq));
+        }
+        h16 mean = f2h(h2f(acc) / h2f(f2h((float)hidden)));
+        h16 me = f2h(h2f(mean) + h2f(f2h(eps)));
+        h16 rs = f2h(1.0f / sqrtf(h2f(me)));
+        for (int i = 0; i < hidden; i++) {
+            h16 n = f2h(h2f(x[i]) * h2f(rs));
+            out[(size_t)t * hidden + i] = f2h(h2f(n) * h2f(w[i]));
+        }
+    }
+}
+
+/* ----------------------------------------------------------- elementwise ---- */
+
+/* siluFunc on the reference's GPU path, tensorLib/src/device/cuda/CUDA.cu:334-342, and the
+ * float branch of the CPU one (tensorLib/src/device/cpu/CPU.cpp:220-223):
+ * half(float(x) * (1/(1+exp(-float(x))))). */
+void tlo_silu_f16(const h16* in, h16* out, size_t n) {
+#pragma omp parallel for
+    for (long i = 0; i < (long)n; i++) {
+        float x = h2f(in[i]);
+        out[i] = f2h(x * (1.0f / (1.0f + expf(-x))));
+    }
+}
+
+/* Literal CPU half branch, tensorLib/src/device/cpu/CPU.cpp:216-219: the exponent has the
+ * wrong sign (x * 1/(1+exp(+x))).  Kept only to document the deviation.  PARITY UNPINNED. */
+void tlo_silu_f16_cpu_literal(const h16* in, h16* out, size_t n) {
+#pragma omp parallel for
+    for (long i = 0; i < (long)n; i++) {
+        float x = h2f(in[i]);
+        h16 sg = f2h(1.0f / (1.0f + expf(x)));
+        out[i] = f2h(x * h2f(sg));
+    }
+}
+
+/* addFunc/subFunc/mulFunc/divFunc on halves, tensorLib/src/device/cpu/CPU.cpp:277-296:
+ * one operator, one rounding.  op: 0 add, 1 sub, 2 mul, 3 div. */
+static inline h16 bin_op(h16 a, h16 b, int op) {
+    float x = h2f(a), y = h2f(b);
+    switch (op) {
+        case 0: return f2h(x + y);
+        case 1: return f2h(x - y);
+        case 2: return f2h(x * y);
+        default: return f2h(x / y);
+    }
+}
+void tlo_binary_f16(const h16* a, const h16* b, h16* out, size_t n, int op) {
+#pragma omp parallel for
+    for (long i = 0; i < (long)n; i++) out[i] = bin_op(a[i], b[i], op);
+}
+/* applyBinaryScalarOperation, tensorLib/src/device/cpu/CPU.cpp:323-337. */
+void tlo_binary_scalar_f16(const h16* a, h16 s, h16* out, size_t n, int op) {
+#pragma omp parallel for
+    for (long i = 0; i < (long)n; i++) out[i] = bin_op(a[i], s, op);
+}
+
+/* silu then multiply, each rounded to half as the two reference ops do
+ * (model/llama2_7b/src/Transformer.cpp:137-141). */
+void tlo_silu_mul_f16(const h16* a, const h16* b, h16* out, size_t n) {
+#pragma omp parallel for
+    for (long i = 0; i < (long)n; i++) {
+        float x = h2f(a[i]);
+        h16 s = f2h(x * (1.0f / (1.0f + expf(-x))));
+        out[i] = f2h(h2f(s) * h2f(b[i]));
+    }
+}
+
+/* ---------------------------------------------------------------- layout ---- */
+
+/* convertIdx, tensorLib/include/device/cpu/CPU.hpp:138-148. */
+static inline size_t convert_idx(size_t lin, const int* shape, const int* stride, int ndim, size_t offset) {
+    size_t r = 0;
+    for (int d = ndim - 1; d >= 0; --d) {
+        size_t id = lin % (size_t)shape[d];
+        lin /= (size_t)shape[d];
+        r += id * (size_t)stride[d];
+    }
+    return r + offset;
+}
+/* CPU<dtype>::contiguous, tensorLib/src/device/cpu/CPU.cpp:127-139. */
+void tlo_contiguous_f16(const h16* base, h16* out, const int* shape, const int* stride, int ndim,
+                        size_t offset, size_t n) {
+#pragma omp parallel for
+    for (long i = 0; i < (long)n; i++) out[i] = base[convert_idx((size_t)i, shape, stride, ndim, offset)];
+}
+/* CPU<dtype>::setItemEwise, tensorLib/src/device/cpu/CPU.cpp:141-154. */
+void tlo_set_item_ewise_f16(h16* base, const h16* src, const int* shape, const int* stride, int ndim,
+                            size_t offset, size_t n) {
+#pragma omp parallel for
+    for (long i = 0; i < (long)n; i++) base[convert_idx((size_t)i, shape, stride, ndim, offset)] = src[i];
+}
+
+/* reduceOperationArg<argmaxFunc>, tensorLib/src/device/cpu/CPU.cpp:356-372: strict '>' so
+ * the first maximum wins. */
+void tlo_argmax_f16(const h16* in, int* out, size_t reduce_size, size_t num_elements) {
+#pragma omp parallel for
+    for (long r = 0; r < (long)(num_elements / reduce_size); r++) {
+        const h16* x = in + (size_t)r * reduce_size;
+        float best = h2f(x[0]);
+        int bi = 0;
+        for (size_t j = 1; j < reduce_size; j++) {
+            float v = h2f(x[j]);
+            if (v > best) { best = v; bi = (int)j; }
+        }
+        out[r] = bi;
+    }
+}
+
+/* Embedding::forward, tensorLib/src/nn/embedding.cpp:47-81: row gather. */
+void tlo_embedding_f16(const h16* table, const int* ids, h16* out, int n_tokens, int dim) {
+    for (int t = 0; t < n_tokens; t++)
+        memcpy(out + (size_t)t * dim, table + (size_t)ids[t] * dim, (size_t)dim * sizeof(h16));
+}

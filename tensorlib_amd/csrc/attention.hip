@@ -1,0 +1,247 @@
+// Attention helpers for the Llama2 driver.
+//
+// tl_decode_attention_f16: single-token attention that reads the KV cache in place.  The
+// reference (model/llama2_7b/src/Transformer.cpp:55-109) re-gathers the whole K and V cache
+// into contiguous scratch every step, then issues 2*n_heads GEMV launches, a scalar divide
+// and a softmax.  Here one launch covers all heads: the T cached positions are cut into
+// chunks, each (head, chunk) workgroup produces a partial (max, sum, weighted V) triple in
+// fp32, and a second tiny launch merges the chunks (the split keeps >= 256 workgroups busy
+// although there are only n_heads independent rows).
+//
+// tl_causal_mask_f16: the additive mask of Transformer::get_mask
+// (model/llama2_7b/src/Transformer.cpp:231-261) written by one kernel instead of one
+// host-to-device copy per element.
+#include <mutex>
+
+#include "tl_internal.h"
+
+namespace tl {
+
+template <int CTRL>
+__device__ __forceinline__ float dppf(float v) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, true));
+}
+
+// Sum over groups of LPR adjacent lanes, LPR in {8,16,32}; all lanes of a group get the sum.
+template <int LPR>
+__device__ __forceinline__ float lanes_sum(float v) {
+    v += dppf<0xB1>(v);
+    v += dppf<0x4E>(v);
+    v += dppf<0x141>(v);
+    if constexpr (LPR >= 16) v += dppf<0x140>(v);
+    if constexpr (LPR == 32) v += __shfl_xor(v, 16, 64);
+    return v;
+}
+
+constexpr int kAttnThreads = 256;
+constexpr int kAttnChunk = 64;  // cached positions per workgroup
+
+// partial layout per (head, chunk): [0] = max, [1] = sum, [2 .. 2+head_dim) = sum_t p_t * V[t]
+template <int LPR>
+__global__ void __launch_bounds__(kAttnThreads)
+decode_attn_partial_kernel(half_t* out, float* partial, const half_t* q, const half_t* cache_k,
+                           const half_t* cache_v, int T, int n_heads, float inv_scale, int n_chunks) {
+    constexpr int D = LPR * 8;
+    constexpr int GROUPS = kAttnThreads / LPR;
+    __shared__ float sc[kAttnChunk];
+    __shared__ float red[16];
+    __shared__ float obuf[GROUPS][D];
+
+    const int h = blockIdx.x;
+    const int chunk = blockIdx.y;
+    const int t0 = chunk * kAttnChunk;
+    const int t1 = (t0 + kAttnChunk < T) ? (t0 + kAttnChunk) : T;
+    const int tid = threadIdx.x;
+    const int sub = tid % LPR;
+    const int grp = tid / LPR;
+    const size_t row_stride = (size_t)n_heads * D;
+
+    const half8_t qv = *reinterpret_cast<const half8_t*>(q + (size_t)h * D + sub * 8);
+
+    // scores
+    for (int t = t0 + grp; t < t1; t += GROUPS) {
+        const half8_t kv = *reinterpret_cast<const half8_t*>(cache_k + (size_t)t * row_stride + (size_t)h * D + sub * 8);
+        float s = 0.f;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) s = __builtin_fmaf((float)qv[i], (float)kv[i], s);
+        s = lanes_sum<LPR>(s);
+        if (sub == 0) sc[t - t0] = s * inv_scale;
+    }
+    __syncthreads();
+
+    // chunk max and sum (kAttnChunk == 64: wavefront 0 alone can reduce it)
+    float m, l;
+    {
+        const int n = t1 - t0;
+        float v = (tid < n) ? sc[tid] : -INFINITY;
+        if (tid < 64) {
+            float mx = v;
+            mx = fmaxf(mx, dppf<0xB1>(mx));
+            mx = fmaxf(mx, dppf<0x4E>(mx));
+            mx = fmaxf(mx, dppf<0x141>(mx));
+            mx = fmaxf(mx, dppf<0x140>(mx));
+            mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+            mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+            const float p = (tid < n) ? expf(v - mx) : 0.f;
+            float sm = p;
+            sm += dppf<0xB1>(sm);
+            sm += dppf<0x4E>(sm);
+            sm += dppf<0x141>(sm);
+            sm += dppf<0x140>(sm);
+            sm += __shfl_xor(sm, 16, 64);
+            sm += __shfl_xor(sm, 32, 64);
+            if (tid < n) sc[tid] = p;
+            if (tid == 0) { red[0] = mx; red[1] = sm; }
+        }
+        __syncthreads();
+        m = red[0];
+        l = red[1];
+    }
+
+    // weighted sum of V rows: thread (grp, sub) accumulates dims [sub*8, sub*8+8) over its positions
+    float acc[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) acc[i] = 0.f;
+    for (int t = t0 + grp; t < t1; t += GROUPS) {
+        const half8_t vv = *reinterpret_cast<const half8_t*>(cache_v + (size_t)t * row_stride + (size_t)h * D + sub * 8);
+        const float p = sc[t - t0];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) acc[i] = __builtin_fmaf(p, (float)vv[i], acc[i]);
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) obuf[grp][sub * 8 + i] = acc[i];
+    __syncthreads();
+    if (tid < D) {
+        float o = 0.f;
+#pragma unroll
+        for (int g = 0; g < GROUPS; ++g) o += obuf[g][tid];
+        if (n_chunks == 1) {
+            out[(size_t)h * D + tid] = (half_t)(o / l);
+        } else {
+            float* p = partial + ((size_t)h * n_chunks + chunk) * (D + 2);
+            p[2 + tid] = o;
+            if (tid == 0) { p[0] = m; p[1] = l; }
+        }
+    }
+}
+
+__global__ void __launch_bounds__(256)
+decode_attn_merge_kernel(half_t* out, const float* partial, int D, int n_chunks) {
+    const int h = blockIdx.x;
+    const int d = threadIdx.x;
+    if (d >= D) return;
+    const float* base = partial + (size_t)h * n_chunks * (D + 2);
+    float m = -INFINITY;
+    for (int c = 0; c < n_chunks; ++c) m = fmaxf(m, base[(size_t)c * (D + 2)]);
+    float l = 0.f, o = 0.f;
+    for (int c = 0; c < n_chunks; ++c) {
+        const float* p = base + (size_t)c * (D + 2);
+        const float w = expf(p[0] - m);
+        l = __builtin_fmaf(p[1], w, l);
+        o = __builtin_fmaf(p[2 + d], w, o);
+    }
+    out[(size_t)h * D + d] = (half_t)(o / l);
+}
+
+// mask[r, i, j] = (j > start_pos + i) ? -inf : 0 for r < reps, i < seqlen, j < start_pos + seqlen
+__global__ void __launch_bounds__(256)
+causal_mask_kernel(half_t* mask, int seqlen, int start_pos, size_t n) {
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    const int cols = start_pos + seqlen;
+    for (size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x; idx < n; idx += stride) {
+        const int j = (int)(idx % cols);
+        const int i = (int)((idx / cols) % seqlen);
+        mask[idx] = (j > start_pos + i) ? (half_t)(-INFINITY) : (half_t)0.f;
+    }
+}
+
+// Library-owned fp32 workspace for the chunk partials, grown on demand.
+static std::mutex g_ws_mu;
+static float* g_ws = nullptr;
+static size_t g_ws_floats = 0;
+
+static int workspace(size_t floats, float** out) {
+    std::lock_guard<std::mutex> lk(g_ws_mu);
+    if (floats > g_ws_floats) {
+        if (g_ws) {
+            TL_HIP_TRY(hipStreamSynchronize(stream()));
+            TL_HIP_TRY(hipFree(g_ws));
+            g_ws = nullptr;
+            g_ws_floats = 0;
+        }
+        size_t want = floats < (1u << 20) ? (1u << 20) : floats;
+        hipError_t e = hipMalloc((void**)&g_ws, want * sizeof(float));
+        if (e != hipSuccess) {
+            (void)hipGetLastError();
+            return set_error(TL_ENOMEM, "attention workspace: hipMalloc(%zu bytes) failed: %s", want * sizeof(float),
+                             hipGetErrorString(e));
+        }
+        g_ws_floats = want;
+    }
+    *out = g_ws;
+    return TL_OK;
+}
+
+}  // namespace tl
+
+extern "C" {
+
+int tl_decode_attention_f16(void* out, const void* q, const void* cache_k, const void* cache_v, int T, int n_heads,
+                            int head_dim) {
+    TL_ENSURE_INIT();
+    TL_REQUIRE(out && q && cache_k && cache_v, "tl_decode_attention_f16: null pointer");
+    TL_REQUIRE(T >= 1 && n_heads >= 1, "tl_decode_attention_f16: bad sizes T=%d n_heads=%d", T, n_heads);
+    TL_REQUIRE(head_dim == 64 || head_dim == 128 || head_dim == 256,
+               "tl_decode_attention_f16: head_dim %d not supported (64, 128 or 256)", head_dim);
+    TL_REQUIRE(tl::aligned16(q) && tl::aligned16(cache_k) && tl::aligned16(cache_v),
+               "tl_decode_attention_f16: q and the caches must be 16-byte aligned");
+    TL_REQUIRE(n_heads <= 65535, "tl_decode_attention_f16: too many heads");
+    const int n_chunks = (T + tl::kAttnChunk - 1) / tl::kAttnChunk;
+    TL_REQUIRE(n_chunks <= 65535, "tl_decode_attention_f16: T=%d too long", T);
+    float* ws = nullptr;
+    if (n_chunks > 1) {
+        int rc = tl::workspace((size_t)n_heads * n_chunks * (head_dim + 2), &ws);
+        if (rc != TL_OK) return rc;
+    }
+    // the reference divides the scores by half(sqrt(head_dim)) (Transformer.cpp:94)
+    const float scale = (float)(tl::half_t)sqrtf((float)head_dim);
+    const float inv_scale = 1.0f / scale;
+    dim3 grid(n_heads, n_chunks);
+    hipStream_t st = tl::stream();
+    if (head_dim == 64)
+        hipLaunchKernelGGL(tl::decode_attn_partial_kernel<8>, grid, dim3(tl::kAttnThreads), 0, st, (tl::half_t*)out, ws,
+                           (const tl::half_t*)q, (const tl::half_t*)cache_k, (const tl::half_t*)cache_v, T, n_heads,
+                           inv_scale, n_chunks);
+    else if (head_dim == 128)
+        hipLaunchKernelGGL(tl::decode_attn_partial_kernel<16>, grid, dim3(tl::kAttnThreads), 0, st, (tl::half_t*)out,
+                           ws, (const tl::half_t*)q, (const tl::half_t*)cache_k, (const tl::half_t*)cache_v, T, n_heads,
+                           inv_scale, n_chunks);
+    else
+        hipLaunchKernelGGL(tl::decode_attn_partial_kernel<32>, grid, dim3(tl::kAttnThreads), 0, st, (tl::half_t*)out,
+                           ws, (const tl::half_t*)q, (const tl::half_t*)cache_k, (const tl::half_t*)cache_v, T, n_heads,
+                           inv_scale, n_chunks);
+    TL_CHECK_LAUNCH("decode_attn_partial_kernel");
+    if (n_chunks > 1) {
+        hipLaunchKernelGGL(tl::decode_attn_merge_kernel, dim3(n_heads), dim3(256), 0, st, (tl::half_t*)out, ws, head_dim,
+                           n_chunks);
+        TL_CHECK_LAUNCH("decode_attn_merge_kernel");
+    }
+    return TL_OK;
+}
+
+int tl_causal_mask_f16(void* mask, int reps, int seqlen, int start_pos) {
+    TL_ENSURE_INIT();
+    TL_REQUIRE(mask, "tl_causal_mask_f16: null pointer");
+    TL_REQUIRE(reps >= 0 && seqlen >= 0 && start_pos >= 0, "tl_causal_mask_f16: negative size");
+    const size_t n = (size_t)reps * seqlen * ((size_t)start_pos + seqlen);
+    if (n == 0) return TL_OK;
+    size_t blocks = (n + 255) / 256;
+    const size_t cap = (size_t)tl::device_info().cu_count * 16;
+    if (blocks > cap) blocks = cap;
+    hipLaunchKernelGGL(tl::causal_mask_kernel, dim3((unsigned)blocks), dim3(256), 0, tl::stream(), (tl::half_t*)mask,
+                       seqlen, start_pos, n);
+    TL_CHECK_LAUNCH("causal_mask_kernel");
+    return TL_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,78 @@
+// Internal helpers shared by the HIP translation units of libtensorlib_amd.so.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <cstdarg>
+#include <cstddef>
+#include <cstdint>
+#include <cstdio>
+
+#include "tensorlib_amd.h"
+
+namespace tl {
+
+typedef _Float16 half_t;
+typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
+typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+typedef float float4_t __attribute__((ext_vector_type(4)));
+typedef float float16_t __attribute__((ext_vector_type(16)));
+
+constexpr int kWave = 64;  // CDNA wavefront width
+
+// Per-thread last-error message; set_error returns `code` so call sites can `return set_error(...)`.
+int set_error(int code, const char* fmt, ...) __attribute__((format(printf, 2, 3)));
+void clear_error();
+
+// Stream all kernels of this library are enqueued on.
+hipStream_t stream();
+
+// Device facts gathered by tl_init (lazily initialised on first use).
+struct DeviceInfo {
+    int ordinal = -1;
+    int cu_count = 0;
+    int wave_size = 0;
+    size_t lds_per_block = 0;
+    char arch[64] = {0};
+};
+const DeviceInfo& device_info();
+int ensure_init();
+
+// out[i] = bits for i < n, as a kernel (safe to record into a HIP graph).
+int launch_fill_f16(void* out, uint16_t bits, size_t n);
+
+// Shared launchers (batch strides in elements; batch == 1 ignores them).
+int launch_gemv(const void* x, const void* W, void* y, size_t N, size_t K, size_t batch, size_t sx,
+                size_t sw, size_t sy);
+int launch_hgemm(const void* A, const void* B, void* C, size_t M, size_t N, size_t K, size_t batch,
+                 size_t sa, size_t sb, size_t sc);
+
+inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+}  // namespace tl
+
+#define TL_HIP_TRY(expr)                                                                        \
+    do {                                                                                        \
+        hipError_t _e = (expr);                                                                 \
+        if (_e != hipSuccess)                                                                   \
+            return tl::set_error(TL_EHIP, "%s failed: %s (%s:%d)", #expr, hipGetErrorString(_e), \
+                                 __FILE__, __LINE__);                                           \
+    } while (0)
+
+// After a kernel launch: surfaces launch-configuration errors without synchronising.
+#define TL_CHECK_LAUNCH(name)                                                                       \
+    do {                                                                                            \
+        hipError_t _e = hipGetLastError();                                                          \
+        if (_e != hipSuccess)                                                                       \
+            return tl::set_error(TL_EHIP, "launch of %s failed: %s", name, hipGetErrorString(_e));  \
+    } while (0)
+
+#define TL_REQUIRE(cond, ...)                                   \
+    do {                                                        \
+        if (!(cond)) return tl::set_error(TL_EINVAL, __VA_ARGS__); \
+    } while (0)
+
+#define TL_ENSURE_INIT()                 \
+    do {                                 \
+        int _rc = tl::ensure_init();     \
+        if (_rc != TL_OK) return _rc;    \
+    } while (0)

@@ -1,0 +1,308 @@
+"""Python mirror of the reference's ``Device<half>`` interface over the C ABI.
+
+Method names and argument meaning follow tensorLib/include/device/Device.hpp:13-101; the
+``matmul`` method follows ``ops::matmul<dtype>::call2`` (tensorLib/src/ops/matmul.cpp:206-324)
+including its error behaviour (``ValueError`` where the reference throws
+``std::invalid_argument``).  Tensors are torch CUDA tensors used purely as device memory:
+every computation happens in libtensorlib_amd.so.
+"""
+from __future__ import annotations
+
+import ctypes
+import math
+
+import numpy as np
+import torch
+
+from ._lib import TensorLibError, check, lib
+
+_OPS = {"add": 0, "sub": 1, "mul": 2, "div": 3}
+
+
+def _ptr(t: torch.Tensor) -> ctypes.c_void_p:
+    return ctypes.c_void_p(t.data_ptr())
+
+
+def _req(t: torch.Tensor, dtype=torch.float16, name="tensor") -> torch.Tensor:
+    if not isinstance(t, torch.Tensor) or not t.is_cuda:
+        raise TensorLibError(f"{name} must be a CUDA(HIP) tensor; there is no CPU path")
+    if t.dtype != dtype:
+        raise TypeError(f"{name} must be {dtype}, got {t.dtype}")
+    if not t.is_contiguous():
+        raise ValueError(f"{name} must be contiguous")
+    return t
+
+
+def _ints(v):
+    return (ctypes.c_int * len(v))(*[int(i) for i in v])
+
+
+def half_bits(x: float) -> int:
+    return int(np.float16(x).view(np.uint16))
+
+
+class HipDevice:
+    """One GPU; all work goes to the library's stream (torch's current stream by default)."""
+
+    def __init__(self, ordinal: int = 0, bind_torch_stream: bool = True):
+        if not torch.cuda.is_available():
+            raise TensorLibError("no HIP device visible: tensorlib_amd has no CPU fallback")
+        self.lib = lib()
+        self.ordinal = ordinal
+        torch.cuda.set_device(ordinal)
+        check(self.lib.tl_init(ordinal), "tl_init")
+        if bind_torch_stream:
+            self.bind_stream(torch.cuda.current_stream())
+        self.device = torch.device("cuda", ordinal)
+
+    # -- runtime ---------------------------------------------------------------------
+    def bind_stream(self, stream: "torch.cuda.Stream | None") -> None:
+        raw = 0 if stream is None else stream.cuda_stream
+        check(self.lib.tl_set_stream(ctypes.c_void_p(raw)), "tl_set_stream")
+
+    def synchronize(self) -> None:
+        check(self.lib.tl_synchronize(), "tl_synchronize")
+
+    @property
+    def cu_count(self) -> int:
+        return int(self.lib.tl_device_cu_count())
+
+    def empty(self, *shape, dtype=torch.float16) -> torch.Tensor:
+        return torch.empty(*shape, dtype=dtype, device=self.device)
+
+    def from_numpy(self, a: np.ndarray) -> torch.Tensor:
+        return torch.from_numpy(np.ascontiguousarray(a)).to(self.device)
+
+    # -- the hot path ----------------------------------------------------------------
+    def matmul2d(self, A: torch.Tensor, B: torch.Tensor, C: torch.Tensor | None = None) -> torch.Tensor:
+        """C[M,N] = A[M,K] . B[N,K]^T (Device.hpp:22)."""
+        _req(A, name="A"), _req(B, name="B")
+        M, K = A.shape
+        N, K2 = B.shape
+        if K != K2:
+            raise ValueError("Shape mismatch: inner dimensions differ")
+        if C is None:
+            C = self.empty(M, N)
+        _req(C, name="C")
+        if tuple(C.shape) != (M, N):
+            raise ValueError("result shape does not match new_shape")
+        check(self.lib.tl_matmul2d_f16(_ptr(A), _ptr(B), _ptr(C), M, N, K), "tl_matmul2d_f16")
+        return C
+
+    def gemv(self, x: torch.Tensor, W: torch.Tensor, y: torch.Tensor | None = None) -> torch.Tensor:
+        _req(x, name="x"), _req(W, name="W")
+        N, K = W.shape
+        if x.numel() != K:
+            raise ValueError("Shape mismatch: x length differs from K")
+        if y is None:
+            y = self.empty(N)
+        _req(y, name="y")
+        check(self.lib.tl_gemv_f16(_ptr(x), _ptr(W), _ptr(y), N, K), "tl_gemv_f16")
+        return y
+
+    def hgemm(self, A: torch.Tensor, B: torch.Tensor, C: torch.Tensor | None = None) -> torch.Tensor:
+        _req(A, name="A"), _req(B, name="B")
+        M, K = A.shape
+        N, K2 = B.shape
+        if K != K2:
+            raise ValueError("Shape mismatch: inner dimensions differ")
+        if C is None:
+            C = self.empty(M, N)
+        _req(C, name="C")
+        check(self.lib.tl_hgemm_f16(_ptr(A), _ptr(B), _ptr(C), M, N, K), "tl_hgemm_f16")
+        return C
+
+    def matmul2d_f32(self, A: torch.Tensor, B: torch.Tensor) -> torch.Tensor:
+        _req(A, torch.float32, "A"), _req(B, torch.float32, "B")
+        M, K = A.shape
+        N, K2 = B.shape
+        if K != K2:
+            raise ValueError("Shape mismatch: inner dimensions differ")
+        C = self.empty(M, N, dtype=torch.float32)
+        check(self.lib.tl_matmul2d_f32(_ptr(A), _ptr(B), _ptr(C), M, N, K), "tl_matmul2d_f32")
+        return C
+
+    def matmul(self, a: torch.Tensor, b: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:
+        """``Tensor::matmul`` semantics: a[..., M, K] @ b[..., K, N] with broadcast batch dims
+        (tensorLib/src/ops/matmul.cpp:206-324).  ``b`` is transposed to the [N, K] operand the
+        boundary wants; for a Linear weight passed as ``W.t()`` no copy is made."""
+        if a.device != b.device:
+            raise ValueError("Tensors must be on the same device.")
+        if a.dim() < 2 or b.dim() < 2:
+            raise ValueError("Tensors must have at least 2 dimensions for matmul.")
+        if a.shape[-1] != b.shape[-2]:
+            raise ValueError("Shape mismatch: the number of columns in the first tensor must match the number "
+                             "of rows in the second tensor.")
+        A = a.contiguous()
+        Bt = b.transpose(-2, -1).contiguous()  # [..., N, K]; a view of a Linear weight stays a view
+        M, K = A.shape[-2:]
+        N = Bt.shape[-2]
+        ab, bb = list(A.shape[:-2]), list(Bt.shape[:-2])
+        nb = max(len(ab), len(bb))
+        ab = [1] * (nb - len(ab)) + ab
+        bb = [1] * (nb - len(bb)) + bb
+        obatch = []
+        for x, y in zip(ab, bb):
+            if x != y and x != 1 and y != 1:
+                raise ValueError("Shape mismatch: the batch dimensions must be broadcastable.")
+            obatch.append(max(x, y))
+        oshape = obatch + [M, N]
+        if out is None:
+            out = self.empty(*oshape)
+        elif list(out.shape) != oshape:
+            raise ValueError("result shape does not match new_shape")
+        _req(out, name="out")
+        batch = int(np.prod(obatch)) if obatch else 1
+        if batch == 1:
+            check(self.lib.tl_matmul2d_f16(_ptr(A), _ptr(Bt), _ptr(out), M, N, K), "tl_matmul2d_f16")
+            return out
+        # one batched launch when each operand is either fully batched or a single matrix
+        a_full, b_full = int(np.prod(ab)) == batch, int(np.prod(bb)) == batch
+        a_one, b_one = int(np.prod(ab)) == 1, int(np.prod(bb)) == 1
+        if (a_full or a_one) and (b_full or b_one):
+            check(self.lib.tl_matmul2d_batched_f16(_ptr(A), _ptr(Bt), _ptr(out), M, N, K, batch,
+                                                   M * K if a_full else 0, N * K if b_full else 0, M * N),
+                  "tl_matmul2d_batched_f16")
+            return out
+        # general broadcast: the reference's per-matrix loop (matmul.cpp:297-321)
+        Ae = A.reshape(ab + [M, K]).expand(obatch + [M, K])
+        Be = Bt.reshape(bb + [N, K]).expand(obatch + [N, K])
+        o3 = out.view(batch, M, N)
+        for i, idx in enumerate(np.ndindex(*obatch)):
+            Ai, Bi = Ae[idx], Be[idx]
+            esz = 2
+            check(self.lib.tl_matmul2d_f16(ctypes.c_void_p(Ai.data_ptr()), ctypes.c_void_p(Bi.data_ptr()),
+                                           ctypes.c_void_p(o3.data_ptr() + i * M * N * esz), M, N, K),
+                  "tl_matmul2d_f16")
+        return out
+
+    # -- small ops --------------------------------------------------------------------
+    def rms_norm(self, x: torch.Tensor, weight: torch.Tensor, eps: float, out: torch.Tensor | None = None):
+        _req(x, name="x"), _req(weight, name="weight")
+        hidden = x.shape[-1]
+        tokens = x.numel() // hidden
+        out = torch.empty_like(x) if out is None else _req(out, name="out")
+        check(self.lib.tl_rms_norm_f16(_ptr(out), _ptr(x), _ptr(weight), eps, hidden, tokens), "tl_rms_norm_f16")
+        return out
+
+    def apply_rotary_emb(self, x: torch.Tensor, start_pos: int, out: torch.Tensor | None = None):
+        _req(x, name="x")
+        if x.dim() != 4:
+            raise ValueError("apply_rotary_emb expects [B, T, n_heads, head_dim]")
+        B, T, H, D = x.shape
+        out = torch.empty_like(x) if out is None else _req(out, name="out")
+        check(self.lib.tl_apply_rotary_emb_f16(_ptr(x), _ptr(out), start_pos, B, T, H, D), "tl_apply_rotary_emb_f16")
+        return out
+
+    def softmax(self, x: torch.Tensor, out: torch.Tensor | None = None):
+        _req(x, name="x")
+        cols = x.shape[-1]
+        rows = x.numel() // cols if cols else 0
+        out = torch.empty_like(x) if out is None else _req(out, name="out")
+        check(self.lib.tl_softmax_f16(_ptr(out), _ptr(x), rows, cols), "tl_softmax_f16")
+        return out
+
+    def silu(self, x: torch.Tensor, out: torch.Tensor | None = None):
+        _req(x, name="x")
+        out = torch.empty_like(x) if out is None else _req(out, name="out")
+        check(self.lib.tl_silu_f16(_ptr(out), _ptr(x), x.numel()), "tl_silu_f16")
+        return out
+
+    def silu_mul(self, a: torch.Tensor, b: torch.Tensor, out: torch.Tensor | None = None):
+        _req(a, name="a"), _req(b, name="b")
+        out = torch.empty_like(a) if out is None else _req(out, name="out")
+        check(self.lib.tl_silu_mul_f16(_ptr(out), _ptr(a), _ptr(b), a.numel()), "tl_silu_mul_f16")
+        return out
+
+    def binary(self, a: torch.Tensor, b, op: str, out: torch.Tensor | None = None):
+        _req(a, name="a")
+        out = torch.empty_like(a) if out is None else _req(out, name="out")
+        if isinstance(b, torch.Tensor):
+            _req(b, name="b")
+            if b.shape != a.shape:
+                raise ValueError("Shape mismatch in elementwise op")
+            check(self.lib.tl_binary_f16(_ptr(out), _ptr(a), _ptr(b), a.numel(), _OPS[op]), "tl_binary_f16")
+        else:
+            check(self.lib.tl_binary_scalar_f16(_ptr(out), _ptr(a), half_bits(b), a.numel(), _OPS[op]),
+                  "tl_binary_scalar_f16")
+        return out
+
+    def add(self, a, b, out=None): return self.binary(a, b, "add", out)
+    def sub(self, a, b, out=None): return self.binary(a, b, "sub", out)
+    def mul(self, a, b, out=None): return self.binary(a, b, "mul", out)
+    def div(self, a, b, out=None): return self.binary(a, b, "div", out)
+
+    def contiguous(self, base: torch.Tensor, shape, stride, offset: int, out: torch.Tensor | None = None):
+        _req(base, name="base")
+        n = int(np.prod(shape))
+        out = self.empty(*shape) if out is None else _req(out, name="out")
+        check(self.lib.tl_contiguous_f16(_ptr(out), _ptr(base), _ints(shape), _ints(stride), len(shape), offset, n),
+              "tl_contiguous_f16")
+        return out
+
+    def set_item_ewise(self, base: torch.Tensor, src: torch.Tensor, shape, stride, offset: int):
+        _req(base, name="base"), _req(src, name="src")
+        n = int(np.prod(shape))
+        check(self.lib.tl_set_item_ewise_f16(_ptr(base), _ptr(src), _ints(shape), _ints(stride), len(shape), offset, n),
+              "tl_set_item_ewise_f16")
+        return base
+
+    def argmax(self, x: torch.Tensor) -> torch.Tensor:
+        _req(x, name="x")
+        reduce_size = x.shape[-1]
+        out = torch.empty(x.shape[:-1], dtype=torch.int32, device=self.device)
+        check(self.lib.tl_argmax_f16(_ptr(out), _ptr(x), reduce_size, x.numel()), "tl_argmax_f16")
+        return out
+
+    def embedding(self, table: torch.Tensor, ids: torch.Tensor) -> torch.Tensor:
+        _req(table, name="table"), _req(ids, torch.int32, "ids")
+        vocab, dim = table.shape
+        out = self.empty(ids.numel(), dim)
+        check(self.lib.tl_embedding_f16(_ptr(out), _ptr(table), _ptr(ids), ids.numel(), dim, vocab), "tl_embedding_f16")
+        return out
+
+    def full(self, out: torch.Tensor, value: float) -> torch.Tensor:
+        _req(out, name="out")
+        check(self.lib.tl_full_f16(_ptr(out), half_bits(value), out.numel()), "tl_full_f16")
+        return out
+
+    def causal_mask(self, reps: int, seqlen: int, start_pos: int) -> torch.Tensor:
+        out = self.empty(reps, seqlen, start_pos + seqlen)
+        check(self.lib.tl_causal_mask_f16(_ptr(out), reps, seqlen, start_pos), "tl_causal_mask_f16")
+        return out
+
+    def decode_attention(self, q: torch.Tensor, cache_k: torch.Tensor, cache_v: torch.Tensor, T: int):
+        """q: [n_heads, head_dim]; caches: [max_seq, n_heads, head_dim]; attends to positions < T."""
+        _req(q, name="q"), _req(cache_k, name="cache_k"), _req(cache_v, name="cache_v")
+        H, D = q.shape
+        if cache_k.shape[1:] != (H, D) or cache_v.shape != cache_k.shape or T > cache_k.shape[0]:
+            raise ValueError("cache shape does not match q / T")
+        out = torch.empty_like(q)
+        check(self.lib.tl_decode_attention_f16(_ptr(out), _ptr(q), _ptr(cache_k), _ptr(cache_v), T, H, D),
+              "tl_decode_attention_f16")
+        return out
+
+    # -- tuning hooks -------------------------------------------------------------------
+    def set_gemv_variant(self, v: int) -> None:
+        check(self.lib.tl_set_gemv_variant(v), "tl_set_gemv_variant")
+
+    def set_hgemm_variant(self, v: int) -> None:
+        check(self.lib.tl_set_hgemm_variant(v), "tl_set_hgemm_variant")
+
+    def gemv_variants(self) -> list[str]:
+        out, i = [], 0
+        while True:
+            n = self.lib.tl_gemv_variant_name(i)
+            if n is None:
+                return out
+            out.append(n.decode())
+            i += 1
+
+    def hgemm_variants(self) -> list[str]:
+        out, i = [], 0
+        while True:
+            n = self.lib.tl_hgemm_variant_name(i)
+            if n is None:
+                return out
+            out.append(n.decode())
+            i += 1

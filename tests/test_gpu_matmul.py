@@ -1,0 +1,233 @@
+"""GPU parity of the matmul hot path (GEMV + HGEMM) against the CPU oracle, through the C ABI.
+
+Gate (north_star): |gpu - cpu| <= 1e-3 + 1e-2 * |cpu| elementwise on the fp16 outputs; the
+integer-valued and unit-vector cases must match bit for bit.
+"""
+import numpy as np
+import pytest
+import torch
+
+from tensorlib_amd import synth
+from tests.conftest import assert_close_f16
+
+pytestmark = pytest.mark.gpu
+
+RTOL, ATOL = 1e-2, 1e-3
+
+# Llama2-7B decode GEMV sweep (N <- K)
+SWEEP = [(4096, 4096), (11008, 4096), (4096, 11008), (32000, 4096)]
+
+
+def _gemv_case(dev, oracle, N, K, seed, variant=0, w_std=0.02):
+    W = synth.normal_f16(seed, (N, K), w_std)
+    x = synth.normal_f16(seed + 1, (K,), 1.0)
+    dev.set_gemv_variant(variant)
+    try:
+        y = dev.gemv(dev.from_numpy(x), dev.from_numpy(W)).cpu().numpy()
+    finally:
+        dev.set_gemv_variant(0)
+    want = oracle.matmul2d(x[None, :], W)[0]
+    assert_close_f16(y, want, RTOL, ATOL, f"gemv {N}<-{K} variant {variant}")
+
+
+def test_gemv_config_single(dev, oracle):
+    """BASELINE config 0: W[4096,4096] ~ N(0,0.02), x ~ N(0,1)."""
+    _gemv_case(dev, oracle, 4096, 4096, seed=100)
+
+
+@pytest.mark.parametrize("N,K", SWEEP)
+def test_gemv_decode_sweep(dev, oracle, N, K):
+    """BASELINE config 1: the four Llama2-7B decode shapes, through matmul2d with M == 1."""
+    W = synth.normal_f16(200 + N % 97, (N, K), 0.02)
+    x = synth.normal_f16(300 + K % 89, (1, K), 1.0)
+    y = dev.matmul2d(dev.from_numpy(x), dev.from_numpy(W)).cpu().numpy()
+    want = oracle.matmul2d(x, W)
+    assert_close_f16(y, want, RTOL, ATOL, f"matmul2d M=1 {N}<-{K}")
+
+
+def test_gemv_every_variant(dev, oracle):
+    names = dev.gemv_variants()
+    assert len(names) > 4
+    for v in range(1, len(names)):
+        for (N, K) in [(4096, 4096), (1024, 11008), (37, 520), (5, 8), (130, 4104)]:
+            _gemv_case(dev, oracle, N, K, seed=400 + v, variant=v)
+
+
+@pytest.mark.parametrize("N,K", [(1, 1), (3, 7), (64, 127), (257, 1001), (100, 128), (33, 64), (1000, 256),
+                                 (128, 1024), (7, 24), (19, 8192), (2, 40000)])
+def test_gemv_ragged_shapes(dev, oracle, N, K):
+    """Shapes off the fast path: K % 8 != 0, short rows (attention's K = 128), x larger than LDS."""
+    _gemv_case(dev, oracle, N, K, seed=500 + N, w_std=0.05)
+
+
+def test_gemv_integer_inputs_bit_exact(dev, oracle):
+    """Integer-valued operands with |sum| < 2048: every fp32 partial sum is exact, so any summation
+    order must give the oracle's bits."""
+    for (N, K) in [(4096, 4096), (4096, 11008), (300, 136)]:
+        W = synth.small_ints_f16(600, (N, K), -2, 2)
+        x = synth.small_ints_f16(601, (K,), -1, 1)
+        y = dev.gemv(dev.from_numpy(x), dev.from_numpy(W)).cpu().numpy()
+        want = oracle.matmul2d(x[None, :], W)[0]
+        assert np.abs(want.astype(np.float32)).max() < 2048
+        assert np.array_equal(y.view(np.uint16), want.view(np.uint16))
+
+
+def test_gemv_unit_vector_selects_column(dev):
+    """x = e_k must return column k of W exactly (catches index/lane mapping mistakes)."""
+    N, K = 512, 4096
+    W = synth.normal_f16(700, (N, K), 1.0)
+    Wd = dev.from_numpy(W)
+    for k in [0, 1, 7, 8, 63, 64, 511, 512, 2047, 4095]:
+        x = np.zeros(K, np.float16)
+        x[k] = 1.0
+        y = dev.gemv(dev.from_numpy(x), Wd).cpu().numpy()
+        assert np.array_equal(y.view(np.uint16), W[:, k].view(np.uint16)), k
+
+
+def test_gemv_unaligned_pointers(dev, oracle):
+    """Operands not 16-byte aligned must take the generic kernel and still be right."""
+    N, K = 50, 264
+    W = synth.normal_f16(710, (N * K + 8,), 0.1)
+    x = synth.normal_f16(711, (K + 8,), 1.0)
+    Wd, xd = dev.from_numpy(W), dev.from_numpy(x)
+    y = dev.gemv(xd[1:K + 1].view(-1), Wd[3:3 + N * K].view(N, K))
+    want = oracle.matmul2d(x[None, 1:K + 1], W[3:3 + N * K].reshape(N, K))[0]
+    assert_close_f16(y.cpu().numpy(), want, RTOL, ATOL, "unaligned gemv")
+
+
+# ------------------------------------------------------------------------------ HGEMM ----
+
+def _hgemm_case(dev, oracle, M, N, K, seed, variant=0, full=True, a_std=1.0, b_std=0.02):
+    A = synth.normal_f16(seed, (M, K), a_std)
+    B = synth.normal_f16(seed + 1, (N, K), b_std)
+    dev.set_hgemm_variant(variant)
+    try:
+        C = dev.hgemm(dev.from_numpy(A), dev.from_numpy(B)).cpu().numpy()
+    finally:
+        dev.set_hgemm_variant(0)
+    what = f"hgemm {M}x{N}x{K} variant {variant}"
+    if full:
+        assert_close_f16(C, oracle.matmul2d(A, B), RTOL, ATOL, what)
+    else:
+        # sampled parity: 8 full rows + 8192 uniformly drawn entries
+        rng = np.random.default_rng(seed)
+        rows = np.unique(np.concatenate([[0, M - 1], rng.integers(0, M, 6)]))
+        assert_close_f16(C[rows], oracle.matmul2d(A[rows], B), RTOL, ATOL, what + " rows")
+        ii, jj = rng.integers(0, M, 8192), rng.integers(0, N, 8192)
+        assert_close_f16(C[ii, jj], oracle.matmul2d_entries(A, B, ii, jj), RTOL, ATOL, what + " entries")
+    return C
+
+
+@pytest.mark.parametrize("M,N,K", [(128, 4096, 4096), (128, 4096, 11008)])
+def test_hgemm_prefill_full_oracle(dev, oracle, M, N, K):
+    _hgemm_case(dev, oracle, M, N, K, seed=800 + K % 13)
+
+
+@pytest.mark.parametrize("M", [128, 512, 2048])
+@pytest.mark.parametrize("N,K", [(4096, 4096), (11008, 4096), (32000, 4096), (4096, 11008)])
+def test_hgemm_prefill_shapes_sampled(dev, oracle, M, N, K):
+    """BASELINE config 2 at full size: oracle on sampled rows and entries."""
+    _hgemm_case(dev, oracle, M, N, K, seed=900 + M + N % 31, full=False)
+
+
+def test_hgemm_every_variant_ragged(dev, oracle):
+    names = dev.hgemm_variants()
+    for v in range(1, len(names)):
+        for (M, N, K) in [(300, 500, 264), (2, 3, 8), (129, 257, 72), (64, 64, 64), (257, 130, 1000)]:
+            _hgemm_case(dev, oracle, M, N, K, seed=1000 + v, variant=v, b_std=0.1)
+
+
+@pytest.mark.parametrize("M,N,K", [(2, 2, 1), (5, 7, 3), (33, 65, 127), (17, 100, 1001), (300, 2, 9)])
+def test_hgemm_unaligned_k(dev, oracle, M, N, K):
+    _hgemm_case(dev, oracle, M, N, K, seed=1100 + K, b_std=0.1)
+
+
+def test_hgemm_integer_inputs_bit_exact(dev, oracle):
+    M, N, K = 256, 384, 512
+    A = synth.small_ints_f16(1200, (M, K), -2, 2)
+    B = synth.small_ints_f16(1201, (N, K), -2, 2)
+    C = dev.hgemm(dev.from_numpy(A), dev.from_numpy(B)).cpu().numpy()
+    want = oracle.matmul2d(A, B)
+    assert np.array_equal(C.view(np.uint16), want.view(np.uint16))
+    ref = (A.astype(np.float64) @ B.astype(np.float64).T)
+    assert np.array_equal(C.astype(np.float64), ref)
+
+
+def test_hgemm_identity(dev):
+    """B = I returns A; A = I returns B^T (catches a transposed operand or tile mapping)."""
+    n = 320
+    A = synth.normal_f16(1300, (200, n), 1.0)
+    eye = np.eye(n, dtype=np.float16)
+    C = dev.hgemm(dev.from_numpy(A), dev.from_numpy(eye)).cpu().numpy()
+    assert np.array_equal(C.view(np.uint16), A.view(np.uint16))
+    B = synth.normal_f16(1301, (136, n), 1.0)
+    C2 = dev.hgemm(dev.from_numpy(eye), dev.from_numpy(B)).cpu().numpy()
+    assert np.array_equal(C2.view(np.uint16), np.ascontiguousarray(B.T).view(np.uint16))
+
+
+# ------------------------------------------------------- batched / Tensor::matmul plumbing ----
+
+def test_batched_attention_shapes(dev, oracle):
+    """The per-head loops of Attention::forward as one batched call: decode (M=1) and prefill."""
+    H, T, D = 32, 200, 128
+    for S in (1, 40):
+        q = synth.normal_f16(1400, (H, S, D), 1.0)
+        keys = synth.normal_f16(1401, (H, T, D), 1.0)
+        sc = dev.matmul(dev.from_numpy(q), dev.from_numpy(keys).transpose(1, 2)).cpu().numpy()
+        want = oracle.matmul2d_batched(q, keys, H, S, T, D, S * D, T * D)
+        assert_close_f16(sc, want, RTOL, ATOL, f"scores S={S}")
+        p = synth.normal_f16(1402, (H, S, T), 0.1)
+        vals_c = synth.normal_f16(1403, (H, D, T), 1.0)  # values_c layout: [H, D, T]
+        o = dev.matmul(dev.from_numpy(p), dev.from_numpy(vals_c).transpose(1, 2)).cpu().numpy()
+        want = oracle.matmul2d_batched(p, vals_c, H, S, D, T, S * T, D * T)
+        assert_close_f16(o, want, RTOL, ATOL, f"p.v S={S}")
+
+
+def test_matmul_broadcast_semantics(dev):
+    """Tensor::matmul batch broadcasting must agree with np.matmul (the reference's own
+    test_batched_matmul, tensorLib/test/python/test_tensor.py:103-121, on fp16 data)."""
+    rng = np.random.default_rng(7)
+    cases = [((3, 4, 5), (5, 6)), ((2, 1, 4, 8), (3, 8, 5)), ((4, 8), (2, 3, 8, 2)), ((2, 3, 7, 16), (2, 3, 16, 9)),
+             ((5, 1, 3, 4), (1, 6, 4, 2))]
+    for sa, sb in cases:
+        a = rng.integers(-3, 4, sa).astype(np.float16)
+        b = rng.integers(-3, 4, sb).astype(np.float16)
+        got = dev.matmul(dev.from_numpy(a), dev.from_numpy(b)).cpu().numpy()
+        want = np.matmul(a.astype(np.float32), b.astype(np.float32))
+        assert got.shape == want.shape
+        assert np.array_equal(got.astype(np.float32), want), (sa, sb)
+
+
+def test_matmul_error_behaviour(dev):
+    a = dev.empty(4, 5)
+    with pytest.raises(ValueError):
+        dev.matmul(a, dev.empty(6, 3))
+    with pytest.raises(ValueError):
+        dev.matmul(dev.empty(5), dev.empty(5, 2))
+    with pytest.raises(ValueError):
+        dev.matmul(dev.empty(2, 4, 5), dev.empty(3, 5, 2))
+    with pytest.raises(ValueError):
+        dev.matmul(a, dev.empty(5, 3), out=dev.empty(4, 4))
+
+
+def test_matmul2d_f32(dev, oracle):
+    rng = np.random.default_rng(11)
+    for (M, N, K) in [(1, 1, 1), (17, 33, 65), (128, 100, 300)]:
+        A = rng.standard_normal((M, K)).astype(np.float32)
+        B = rng.standard_normal((N, K)).astype(np.float32)
+        C = dev.matmul2d_f32(dev.from_numpy(A), dev.from_numpy(B)).cpu().numpy()
+        np.testing.assert_allclose(C, oracle.matmul2d_f32(A, B), rtol=1e-4, atol=1e-4)
+
+
+def test_linearity_at_full_size(dev):
+    """Size-independent property at the largest decode shape: W.(x1 + x2) == W.x1 + W.x2 for
+    integer-valued operands (exact in fp32)."""
+    N, K = 32000, 4096
+    W = synth.small_ints_f16(1500, (N, K), -2, 2)
+    x1 = synth.small_ints_f16(1501, (K,), -1, 1)
+    x2 = synth.small_ints_f16(1502, (K,), -1, 1)
+    Wd = dev.from_numpy(W)
+    y1 = dev.gemv(dev.from_numpy(x1), Wd).float()
+    y2 = dev.gemv(dev.from_numpy(x2), Wd).float()
+    y12 = dev.gemv(dev.from_numpy((x1 + x2).astype(np.float16)), Wd).float()
+    assert torch.equal(y12, y1 + y2)

@@ -1,0 +1,190 @@
+"""GPU parity of the small kernels around the matmuls (RMSNorm, RoPE, softmax, SiLU,
+elementwise, strided copies, argmax, embedding, mask, fused decode attention) against the
+CPU oracle, through the C ABI.  Floating point: rtol 1e-2 / atol 1e-3 (north_star);
+copies, argmax and embedding: bit-exact."""
+import numpy as np
+import pytest
+import torch
+
+from tensorlib_amd import synth
+from tests.conftest import assert_close_f16
+
+pytestmark = pytest.mark.gpu
+RTOL, ATOL = 1e-2, 1e-3
+
+
+@pytest.mark.parametrize("tokens,hidden", [(1, 4096), (7, 4096), (128, 1024), (3, 100), (5, 8), (2, 11008)])
+def test_rms_norm(dev, oracle, tokens, hidden):
+    x = synth.normal_f16(10, (tokens, hidden), 1.0)
+    w = synth.normal_f16(11, (hidden,), 1.0)
+    got = dev.rms_norm(dev.from_numpy(x), dev.from_numpy(w), 1e-5).cpu().numpy()
+    assert_close_f16(got, oracle.rms_norm(x, w, 1e-5, "fused"), RTOL, ATOL, "rms_norm vs fused semantics")
+    assert_close_f16(got, oracle.rms_norm(x, w, 1e-5, "exact"), RTOL, ATOL, "rms_norm vs float64 definition")
+
+
+def test_rms_norm_in_place(dev, oracle):
+    x = synth.normal_f16(12, (4, 4096), 2.0)
+    w = synth.normal_f16(13, (4096,), 1.0)
+    xd = dev.from_numpy(x)
+    dev.rms_norm(xd, dev.from_numpy(w), 1e-5, out=xd)
+    assert_close_f16(xd.cpu().numpy(), oracle.rms_norm(x, w, 1e-5, "exact"), RTOL, ATOL, "rms_norm in place")
+
+
+@pytest.mark.parametrize("B,T,H,D,start", [(1, 1, 32, 128, 0), (1, 1, 32, 128, 1023), (7, 9, 32, 128, 5),
+                                           (1, 512, 32, 128, 0), (2, 3, 4, 64, 2047), (1, 2, 1, 2, 3)])
+def test_rope(dev, oracle, B, T, H, D, start):
+    x = synth.normal_f16(20, (B, T, H, D), 1.0)
+    got = dev.apply_rotary_emb(dev.from_numpy(x), start).cpu().numpy()
+    assert_close_f16(got, oracle.rope(x, start), RTOL, 2e-3, "rope")
+    xd = dev.from_numpy(x)
+    dev.apply_rotary_emb(xd, start, out=xd)  # in place, as Attention::forward does
+    assert np.array_equal(xd.cpu().numpy().view(np.uint16), got.view(np.uint16))
+
+
+@pytest.mark.parametrize("rows,cols", [(32, 1), (32, 1024), (32, 1025), (3, 5), (32 * 64, 512), (1, 32000), (4, 64),
+                                       (4, 65), (2, 129)])
+def test_softmax(dev, oracle, rows, cols):
+    x = synth.normal_f16(30, (rows, cols), 2.0)
+    got = dev.softmax(dev.from_numpy(x)).cpu().numpy()
+    assert_close_f16(got, oracle.softmax(x), RTOL, ATOL, "softmax")
+    s = got.astype(np.float64).sum(axis=1)
+    assert np.all(np.abs(s - 1.0) < 5e-3)
+
+
+def test_softmax_with_mask_rows(dev, oracle):
+    """-inf entries (the causal mask) give exact zeros; in-place call."""
+    x = synth.normal_f16(31, (16, 40), 1.0)
+    x[:, 25:] = -np.inf
+    xd = dev.from_numpy(x)
+    dev.softmax(xd, out=xd)
+    got = xd.cpu().numpy()
+    assert np.all(got[:, 25:] == 0)
+    assert_close_f16(got, oracle.softmax(x), RTOL, ATOL, "masked softmax")
+
+
+@pytest.mark.parametrize("n", [1, 7, 8, 11008, 11008 * 3 + 5])
+def test_silu_and_silu_mul(dev, oracle, n):
+    a = synth.normal_f16(40, (n,), 3.0)
+    b = synth.normal_f16(41, (n,), 1.0)
+    assert_close_f16(dev.silu(dev.from_numpy(a)).cpu().numpy(), oracle.silu(a), RTOL, ATOL, "silu")
+    assert_close_f16(dev.silu_mul(dev.from_numpy(a), dev.from_numpy(b)).cpu().numpy(), oracle.silu_mul(a, b), RTOL, ATOL,
+                     "silu_mul")
+
+
+@pytest.mark.parametrize("op", ["add", "sub", "mul", "div"])
+def test_binary_bit_exact(dev, oracle, op):
+    """One IEEE operation, one rounding: must equal the oracle bit for bit."""
+    for n in (1, 9, 4096, 11008 + 3):
+        a = synth.normal_f16(50, (n,), 2.0)
+        b = synth.normal_f16(51, (n,), 2.0)
+        got = dev.binary(dev.from_numpy(a), dev.from_numpy(b), op).cpu().numpy()
+        assert np.array_equal(got.view(np.uint16), oracle.binary(a, b, op).view(np.uint16)), (op, n)
+        s = float(np.float16(np.sqrt(128.0)))
+        got = dev.binary(dev.from_numpy(a), s, op).cpu().numpy()
+        assert np.array_equal(got.view(np.uint16), oracle.binary_scalar(a, s, op).view(np.uint16)), (op, n, "scalar")
+
+
+def test_binary_unaligned(dev, oracle):
+    a = synth.normal_f16(52, (1000,), 1.0)
+    b = synth.normal_f16(53, (1000,), 1.0)
+    ad, bd = dev.from_numpy(a), dev.from_numpy(b)
+    out = dev.empty(1000)
+    # unaligned pointers: slices of a larger buffer
+    r = dev.add(ad[1:998], bd[3:1000], out=out[1:998])
+    assert np.array_equal(r.cpu().numpy().view(np.uint16), oracle.binary(a[1:998], b[3:1000], "add").view(np.uint16))
+
+
+def test_contiguous_and_set_item_kv_cache_patterns(dev, oracle):
+    """The strided moves of Attention::forward (Transformer.cpp:49-80): cache write at a
+    position, K gather to [H,T,D], V gather to [H,D,T], q/o transposes."""
+    S, H, D, T = 64, 8, 128, 37
+    cache = synth.normal_f16(60, (S, H, D), 1.0)
+    cd = dev.from_numpy(cache)
+    # keys: cache[:T] viewed [T,H,D] -> transpose(0,1) -> contiguous [H,T,D]
+    got = dev.contiguous(cd, (H, T, D), (D, H * D, 1), 0).cpu().numpy()
+    assert np.array_equal(got.view(np.uint16), np.ascontiguousarray(cache[:T].transpose(1, 0, 2)).view(np.uint16))
+    assert np.array_equal(got.view(np.uint16), oracle.contiguous(cache, (H, T, D), (D, H * D, 1), 0).view(np.uint16))
+    # values: -> [H,D,T] (last dim strided: scalar path)
+    got = dev.contiguous(cd, (H, D, T), (D, 1, H * D), 0).cpu().numpy()
+    assert np.array_equal(got.view(np.uint16), np.ascontiguousarray(cache[:T].transpose(1, 2, 0)).view(np.uint16))
+    # offset + slice: rows 5..9 of the cache
+    got = dev.contiguous(cd, (4, H, D), (H * D, D, 1), 5 * H * D).cpu().numpy()
+    assert np.array_equal(got.view(np.uint16), cache[5:9].view(np.uint16))
+    # setItem: write new k at positions [10, 13)
+    src = synth.normal_f16(61, (3, H, D), 1.0)
+    dev.set_item_ewise(cd, dev.from_numpy(src), (3, H, D), (H * D, D, 1), 10 * H * D)
+    want = oracle.set_item_ewise(cache, src, (3, H, D), (H * D, D, 1), 10 * H * D)
+    assert np.array_equal(cd.cpu().numpy().view(np.uint16), want.view(np.uint16))
+    # odd sizes / broadcast stride 0
+    base = synth.normal_f16(62, (5, 7), 1.0)
+    got = dev.contiguous(dev.from_numpy(base), (3, 5, 7), (0, 7, 1), 0).cpu().numpy()
+    assert np.array_equal(got.view(np.uint16), np.broadcast_to(base, (3, 5, 7)).copy().view(np.uint16))
+
+
+def test_strided_rejects_bad_arguments(dev):
+    from tensorlib_amd import TensorLibError
+    base = dev.empty(64)
+    with pytest.raises(TensorLibError):   # more than 8 dimensions
+        dev.contiguous(base, (1,) * 9, (1,) * 9, 0)
+    with pytest.raises(TensorLibError):   # negative stride
+        dev.contiguous(base, (4,), (-1,), 8)
+
+
+def test_argmax_first_max_wins(dev, oracle):
+    x = synth.normal_f16(70, (5, 32000), 1.0)
+    x[1, 100] = x[1, 31999] = 9.0     # tie: first index must win
+    x[2, :] = 0.5                      # all equal -> 0
+    x[3, 31999] = 20.0                 # max at the very end
+    got = dev.argmax(dev.from_numpy(x)).cpu().numpy()
+    want = oracle.argmax(x)
+    assert np.array_equal(got, want)
+    assert np.array_equal(got, np.argmax(x.astype(np.float32), axis=-1))
+    small = synth.normal_f16(71, (300, 7), 1.0)
+    assert np.array_equal(dev.argmax(dev.from_numpy(small)).cpu().numpy(), oracle.argmax(small))
+
+
+def test_embedding(dev, oracle):
+    table = synth.normal_f16(80, (1000, 4096), 1.0)
+    ids = synth.token_ids(81, 33, 1000)
+    got = dev.embedding(dev.from_numpy(table), dev.from_numpy(ids)).cpu().numpy()
+    assert np.array_equal(got.view(np.uint16), oracle.embedding(table, ids).view(np.uint16))
+    t2 = synth.normal_f16(82, (10, 13), 1.0)
+    ids2 = np.array([9, 0, 3], np.int32)
+    got = dev.embedding(dev.from_numpy(t2), dev.from_numpy(ids2)).cpu().numpy()
+    assert np.array_equal(got.view(np.uint16), t2[ids2].view(np.uint16))
+
+
+def test_full_and_causal_mask(dev):
+    out = dev.empty(1001)
+    dev.full(out, -2.5)
+    assert torch.all(out == -2.5)
+    m = dev.causal_mask(3, 4, 5).cpu().numpy().astype(np.float32)
+    for i in range(4):
+        for j in range(9):
+            want = -np.inf if j > 5 + i else 0.0
+            assert np.all(m[:, i, j] == want)
+
+
+def _attention_chain_oracle(oracle, q, ck, cv, T):
+    """Attention::forward at seqlen 1 composed from CPU-backend ops, in the reference's order
+    (model/llama2_7b/src/Transformer.cpp:84-109): per-head q.K^T (matmul2d, rounded to half),
+    ScalarDiv by half(sqrt(head_dim)), softmax, scores.V (matmul2d)."""
+    H, D = q.shape
+    keys = np.ascontiguousarray(ck[:T].transpose(1, 0, 2))      # [H,T,D]
+    vals = np.ascontiguousarray(cv[:T].transpose(1, 2, 0))      # [H,D,T]
+    sc = oracle.matmul2d_batched(q.reshape(H, 1, D), keys, H, 1, T, D, D, T * D).reshape(H, T)
+    sc = oracle.binary_scalar(sc, np.sqrt(np.float32(D)), "div")
+    p = oracle.softmax(sc)
+    return oracle.matmul2d_batched(p.reshape(H, 1, T), vals, H, 1, D, T, T, D * T).reshape(H, D)
+
+
+@pytest.mark.parametrize("T,H,D", [(1, 32, 128), (5, 32, 128), (64, 32, 128), (65, 32, 128), (1024, 32, 128),
+                                   (2047, 32, 128), (300, 4, 64), (130, 2, 256)])
+def test_decode_attention_fused_vs_chain(dev, oracle, T, H, D):
+    S = max(T, 8)
+    q = synth.normal_f16(90, (H, D), 1.0)
+    ck = synth.normal_f16(91, (S, H, D), 1.0)
+    cv = synth.normal_f16(92, (S, H, D), 1.0)
+    got = dev.decode_attention(dev.from_numpy(q), dev.from_numpy(ck), dev.from_numpy(cv), T).cpu().numpy()
+    want = _attention_chain_oracle(oracle, q, ck, cv, T)
+    assert_close_f16(got, want, RTOL, 2e-3, f"decode attention T={T}")
