@@ -1,0 +1,227 @@
+#!/usr/bin/env python3
+"""Headline benchmark: fp16 GEMV bandwidth over the Llama2-7B decode sweep on one MI355X.
+
+A step is one pass of the hot path over the four decode shapes (N<-K): 4096<-4096 (wq/wk/wv/wo),
+11008<-4096 (w1/w3), 4096<-11008 (w2, split-K) and 32000<-4096 (classifier), each through
+tl_matmul2d_f16 with M == 1.  Inputs are resident in HBM before the timed region; weights rotate
+over several buffer sets (> 1 GB in total) so every launch streams W from HBM, not from the
+256 MB Infinity Cache.
+
+Prints ONE JSON line.  `value` = algorithmic bytes of a step / wall time of a step (GB/s,
+decimal).  `roofline` = the GEMV kernel against the 8 TB/s HBM peak, from a HIP event pair
+recorded on the launch stream around the timed region.  `cpu_baseline` = the CPU oracle
+(a port of the reference's OpenMP CPU<half>::matmul2d) timed on this host on the same sweep.
+`extra` carries per-shape GEMV numbers, prefill HGEMM TFLOP/s and, when the C++ driver is
+built, Llama2-7B decode tok/s.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
+MFMA_FP16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16 MFMA, published
+
+SWEEP = [(4096, 4096), (11008, 4096), (4096, 11008), (32000, 4096)]
+# prefill shapes reported in `extra` (M, N, K)
+HGEMM_SHAPES = [(2048, 4096, 4096), (2048, 11008, 4096), (2048, 32000, 4096), (2048, 4096, 11008),
+                (512, 4096, 4096), (512, 11008, 4096), (512, 32000, 4096), (512, 4096, 11008),
+                (128, 4096, 4096), (128, 11008, 4096), (128, 32000, 4096), (128, 4096, 11008)]
+
+# HBM bytes per GEMV launch measured with rocprofv3 --pmc (FETCH_SIZE, WRITE_SIZE), averaged over
+# the four sweep launches and scaled by the same counters' reading for a copy kernel of known
+# size; None until the counter profile under profiles/ exists.
+GEMV_TRAFFIC_BYTES_PER_LAUNCH = None
+
+
+def parse_args():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--no-extra", action="store_true", help="skip the HGEMM / per-shape / model extras")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    return ap.parse_args()
+
+
+def cpu_baseline(budget_s: float = 10.0):
+    """Time the CPU oracle on the full decode sweep (all four shapes, every row)."""
+    import numpy as np
+    from oracle import oracle
+    from tensorlib_amd import synth
+    mats = []
+    for i, (N, K) in enumerate(SWEEP):
+        mats.append((synth.normal_f16(10 + i, (N, K), 0.02), synth.normal_f16(20 + i, (1, K), 1.0)))
+    oracle.matmul2d(mats[0][1], mats[0][0])  # warm-up (thread pool, tables)
+    times = []
+    t_start = time.perf_counter()
+    while len(times) < 3 or (time.perf_counter() - t_start < budget_s and len(times) < 50):
+        t0 = time.perf_counter()
+        for W, x in mats:
+            oracle.matmul2d(x, W)
+        times.append(time.perf_counter() - t0)
+    med = float(np.median(times))
+    total_bytes = sum(synth.gemv_bytes(N, K) for N, K in SWEEP)
+    return {
+        "value": round(total_bytes / med / 1e9, 3),
+        "unit": "GB/s",
+        "cores": oracle.max_threads(),
+        "kind": "port",
+        "sample": f"full decode sweep (4 GEMVs, {total_bytes} B), median of {len(times)} passes, "
+                  f"{med * 1e3:.1f} ms per pass",
+    }
+
+
+def time_region(fn, reps: int, torch):
+    """Run fn() reps times between a HIP event pair on the current (= library) stream; returns
+    (wall seconds, event seconds)."""
+    e0 = torch.cuda.Event(enable_timing=True)
+    e1 = torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    e0.record()
+    for _ in range(reps):
+        fn()
+    e1.record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    return wall, e0.elapsed_time(e1) * 1e-3
+
+
+def main():
+    args = parse_args()
+    if args.gpus != 1:
+        print(f"bench.py measures one GPU only (every box of this build has one); got --gpus {args.gpus}",
+              file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    from tensorlib_amd import HipDevice, synth
+
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU: tensorlib_amd has no CPU fallback", file=sys.stderr)
+        sys.exit(1)
+    dev = HipDevice(0)
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(1234)
+
+    def randn(shape, std):
+        return (torch.randn(shape, generator=gen, device="cuda", dtype=torch.float32) * std).to(torch.float16)
+
+    # ---- weights: NSETS rotating sets of the four matrices (3 x 476 MB) ------------------
+    NSETS = 3
+    sets = []
+    for _ in range(NSETS):
+        sets.append([(randn((N, K), 0.02), randn((1, K), 1.0), torch.empty((1, N), device="cuda", dtype=torch.float16))
+                     for (N, K) in SWEEP])
+    step_bytes = sum(synth.gemv_bytes(N, K) for N, K in SWEEP)
+    counter = [0]
+
+    def step():
+        s = sets[counter[0] % NSETS]
+        counter[0] += 1
+        for W, x, y in s:
+            dev.matmul2d(x, W, y)
+
+    for _ in range(args.warmup):
+        step()
+    wall, ev = time_region(step, args.steps, torch)
+    ms_per_step = wall * 1e3 / args.steps
+    value = step_bytes / (wall / args.steps) / 1e9
+    launches = args.steps * len(SWEEP)
+    avg_launch_s = ev / launches
+    achieved = (step_bytes / len(SWEEP)) / avg_launch_s / 1e9
+
+    out = {
+        "metric": "fp16 GEMV GB/s (Llama2-7B decode sweep)",
+        "value": round(value, 2),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 5),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f16",
+        "data": "synthetic",
+        "config": {"workload": "Llama2-7B decode GEMV sweep, batch 1 fp16: 4096<-4096, 11008<-4096, 4096<-11008, "
+                               "32000<-4096; W~N(0,0.02), x~N(0,1); fp32 accumulate; weights rotated over "
+                               f"{NSETS} sets ({NSETS * step_bytes / 1e6:.0f} MB)",
+                   "bytes_per_step": step_bytes},
+        "roofline": {
+            "bound": "hbm",
+            "achieved": round(achieved, 2),
+            "peak": HBM_PEAK_GBS,
+            "unit": "GB/s",
+            "frac": round(achieved / HBM_PEAK_GBS, 4),
+            "traffic": GEMV_TRAFFIC_BYTES_PER_LAUNCH,
+            "kernel": "gemv_f16_wave_kernel",
+            "bytes_per_launch": step_bytes / len(SWEEP),
+            "avg_launch_us": round(avg_launch_s * 1e6, 3),
+        },
+    }
+
+    extra = {}
+    if not args.no_extra:
+        # per-shape GEMV, each over >1 GB of rotating weights
+        per_shape = {}
+        for (N, K) in SWEEP:
+            nbuf = max(2, int(1.0e9 // (N * K * 2)) + 1)
+            Ws = [randn((N, K), 0.02) for _ in range(nbuf)]
+            x = randn((1, K), 1.0)
+            y = torch.empty((1, N), device="cuda", dtype=torch.float16)
+            idx = [0]
+
+            def one():
+                dev.matmul2d(x, Ws[idx[0] % nbuf], y)
+                idx[0] += 1
+            for _ in range(10):
+                one()
+            _, ev1 = time_region(one, 200, torch)
+            us = ev1 / 200 * 1e6
+            gbs = synth.gemv_bytes(N, K) / us / 1e3
+            per_shape[f"{N}x{K}"] = {"us": round(us, 2), "GB/s": round(gbs, 1), "frac_hbm": round(gbs / HBM_PEAK_GBS, 4)}
+            del Ws
+        extra["gemv_per_shape"] = per_shape
+        torch.cuda.empty_cache()
+
+        hg = {}
+        for (M, N, K) in HGEMM_SHAPES:
+            A = randn((M, K), 1.0)
+            B = randn((N, K), 0.02)
+            C = torch.empty((M, N), device="cuda", dtype=torch.float16)
+            for _ in range(3):
+                dev.matmul2d(A, B, C)
+            reps = 20
+            _, ev1 = time_region(lambda: dev.matmul2d(A, B, C), reps, torch)
+            us = ev1 / reps * 1e6
+            tf = synth.gemm_flops(M, N, K) / us / 1e6
+            ai = synth.gemm_flops(M, N, K) / synth.gemm_min_bytes(M, N, K)
+            bound_tf = min(MFMA_FP16_PEAK_TFLOPS, ai * HBM_PEAK_GBS / 1e3)
+            hg[f"{M}x{N}x{K}"] = {"us": round(us, 1), "TFLOP/s": round(tf, 1),
+                                  "frac_mfma_peak": round(tf / MFMA_FP16_PEAK_TFLOPS, 4),
+                                  "bound": "mfma" if bound_tf >= MFMA_FP16_PEAK_TFLOPS else "hbm",
+                                  "frac_of_bound": round(tf / bound_tf, 4)}
+        extra["hgemm_prefill"] = hg
+        try:
+            from tensorlib_amd import llama2
+            extra["llama2_7b_decode"] = llama2.bench_decode(dev)
+        except ImportError:
+            pass
+    out["extra"] = extra
+
+    if not args.no_cpu:
+        out["cpu_baseline"] = cpu_baseline()
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

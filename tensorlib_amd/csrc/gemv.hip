@@ -11,6 +11,8 @@
 //     (used for the 11008-wide down-projection); partial sums meet in LDS, in a fixed order;
 //   * the 64 partial sums of a wavefront are combined with DPP row operations and
 //     four v_readlane, no LDS traffic.
+#include <cstring>
+
 #include "tl_internal.h"
 
 namespace tl {
@@ -182,6 +184,120 @@ __global__ void __launch_bounds__(WAVES * 64) gemv_f16_wave_kernel(GemvArgs a) {
     }
 }
 
+// Single-tile streaming kernel: the K segment of a wavefront fits one register tile
+// (segment <= 64*UNROLL chunks), so the chunk a lane owns is fixed for the whole kernel, the
+// matching piece of x is read once and kept in registers, and row blocks are double buffered:
+// the loads of row block i+1 are in flight while block i is reduced.
+//   XMODE 0: x goes global -> LDS (whole vector, once per workgroup) -> registers;
+//            the first W tile is requested before the staging barrier.
+//   XMODE 1: every wavefront reads its own K segment of x straight into registers.
+// Dynamic LDS: [K8 chunks of x when XMODE == 0] + 2*RG*KSPLIT*ROWS floats when KSPLIT > 1.
+template <int WAVES, int ROWS, int UNROLL, int KSPLIT, int XMODE>
+__global__ void __launch_bounds__(WAVES * 64) gemv_f16_stream_kernel(GemvArgs a) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+    half8_t* xs = reinterpret_cast<half8_t*>(smem_raw);
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int batch = blockIdx.y;
+    const half8_t* __restrict__ x = a.x + (size_t)batch * a.sx8;
+    const half8_t* __restrict__ W = a.W + (size_t)batch * a.sw8;
+    half_t* __restrict__ y = a.y + (size_t)batch * a.sy;
+    const int K8 = a.K8;
+    const int N = a.N;
+
+    constexpr int RG = WAVES / KSPLIT;
+    const int kpart = wave % KSPLIT;
+    const int rgrp = wave / KSPLIT;
+    const int seg = (K8 + KSPLIT - 1) / KSPLIT;
+    const int c0 = kpart * seg;
+    const int c1 = (c0 + seg < K8) ? (c0 + seg) : K8;
+    float* part = reinterpret_cast<float*>(xs + (XMODE == 0 ? K8 : 0));  // [2][RG][KSPLIT][ROWS]
+
+    int cidx[UNROLL];
+    bool ok[UNROLL];
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+        cidx[u] = c0 + u * 64 + lane;
+        ok[u] = cidx[u] < c1;
+    }
+    const half8_t zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+
+    half8_t xv[UNROLL];
+    if constexpr (XMODE == 1) {
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u) xv[u] = ok[u] ? x[cidx[u]] : zero8;
+    }
+
+    half8_t cur[ROWS][UNROLL], nxt[ROWS][UNROLL];
+    auto load_tile = [&](half8_t (&t)[ROWS][UNROLL], int rb) {
+        const int row0 = (rb * RG + rgrp) * ROWS;
+#pragma unroll
+        for (int r = 0; r < ROWS; ++r) {
+            int row = row0 + r;
+            row = row < N ? row : N - 1;
+            const half8_t* wr = W + (size_t)row * K8;
+#pragma unroll
+            for (int u = 0; u < UNROLL; ++u) t[r][u] = ok[u] ? __builtin_nontemporal_load(wr + cidx[u]) : zero8;
+        }
+    };
+
+    int rb = blockIdx.x;
+    if (rb < a.num_row_blocks) load_tile(cur, rb);
+
+    if constexpr (XMODE == 0) {
+        for (int c = tid; c < K8; c += WAVES * 64) xs[c] = x[c];
+        __syncthreads();
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u) xv[u] = xs[ok[u] ? cidx[u] : 0];
+    }
+
+    int it = 0;
+    for (; rb < a.num_row_blocks; rb += gridDim.x, ++it) {
+        const int nrb = rb + gridDim.x;
+        const bool has_next = nrb < a.num_row_blocks;
+        if (has_next) load_tile(nxt, nrb);
+
+        float acc[ROWS];
+#pragma unroll
+        for (int r = 0; r < ROWS; ++r) {
+            acc[r] = 0.f;
+#pragma unroll
+            for (int u = 0; u < UNROLL; ++u) acc[r] = dot8(cur[r][u], xv[u], acc[r]);
+            acc[r] = wave_sum(acc[r]);
+        }
+        const int row0 = (rb * RG + rgrp) * ROWS;
+        if constexpr (KSPLIT == 1) {
+            if (lane < ROWS) {
+                float v = acc[0];
+#pragma unroll
+                for (int r = 1; r < ROWS; ++r) v = (lane == r) ? acc[r] : v;
+                if (row0 + lane < N) y[row0 + lane] = (half_t)v;
+            }
+        } else {
+            float* p = part + (it & 1) * (RG * KSPLIT * ROWS);
+            if (lane == 0) {
+#pragma unroll
+                for (int r = 0; r < ROWS; ++r) p[(rgrp * KSPLIT + kpart) * ROWS + r] = acc[r];
+            }
+            __syncthreads();
+            if (kpart == 0 && lane < ROWS) {
+                float v = 0.f;
+#pragma unroll
+                for (int s = 0; s < KSPLIT; ++s) v += p[(rgrp * KSPLIT + s) * ROWS + lane];
+                if (row0 + lane < N) y[row0 + lane] = (half_t)v;
+            }
+        }
+        if (has_next) {
+#pragma unroll
+            for (int r = 0; r < ROWS; ++r)
+#pragma unroll
+                for (int u = 0; u < UNROLL; ++u) cur[r][u] = nxt[r][u];
+        }
+    }
+}
+
 // Short rows (K8 < 64 chunks): LPR lanes per row, 64/LPR rows per wavefront pass; x read
 // straight from global memory (it is at most 1 KiB).  Serves attention's q.K^T (K = 128).
 template <int LPR>
@@ -233,37 +349,79 @@ gemv_f16_generic_kernel(const half_t* __restrict__ x0, const half_t* __restrict_
 struct GemvVariant {
     const char* name;
     int waves, rows, unroll, ksplit;
+    int xmode;  // -1: looping kernel (any K), 0/1: single-tile streaming kernel
     void (*kernel)(GemvArgs);
 };
 
+#define TL_LOOP(W_, R_, U_, S_, NT_) \
+    { "loop_w" #W_ "r" #R_ "u" #U_ "s" #S_ "nt" #NT_, W_, R_, U_, S_, -1, gemv_f16_wave_kernel<W_, R_, U_, S_, NT_> }
+#define TL_STREAM(W_, R_, U_, S_, X_) \
+    { "stream_w" #W_ "r" #R_ "u" #U_ "s" #S_ "x" #X_, W_, R_, U_, S_, X_, gemv_f16_stream_kernel<W_, R_, U_, S_, X_> }
+#define TL_STREAM2(W_, R_, U_, S_) TL_STREAM(W_, R_, U_, S_, 0), TL_STREAM(W_, R_, U_, S_, 1)
+
 static const GemvVariant g_variants[] = {
-    {"auto", 0, 0, 0, 0, nullptr},
-    {"w4r2u4s1", 4, 2, 4, 1, gemv_f16_wave_kernel<4, 2, 4, 1, false>},     // 1
-    {"w4r2u8s1", 4, 2, 8, 1, gemv_f16_wave_kernel<4, 2, 8, 1, false>},     // 2
-    {"w4r4u8s1", 4, 4, 8, 1, gemv_f16_wave_kernel<4, 4, 8, 1, false>},     // 3
-    {"w4r1u8s1", 4, 1, 8, 1, gemv_f16_wave_kernel<4, 1, 8, 1, false>},     // 4
-    {"w4r4u4s1", 4, 4, 4, 1, gemv_f16_wave_kernel<4, 4, 4, 1, false>},     // 5
-    {"w8r2u8s1", 8, 2, 8, 1, gemv_f16_wave_kernel<8, 2, 8, 1, false>},     // 6
-    {"w4r2u4s2", 4, 2, 4, 2, gemv_f16_wave_kernel<4, 2, 4, 2, false>},     // 7
-    {"w4r2u6s4", 4, 2, 6, 4, gemv_f16_wave_kernel<4, 2, 6, 4, false>},     // 8
-    {"w4r4u6s4", 4, 4, 6, 4, gemv_f16_wave_kernel<4, 4, 6, 4, false>},     // 9
-    {"w8r2u6s4", 8, 2, 6, 4, gemv_f16_wave_kernel<8, 2, 6, 4, false>},     // 10
-    {"w4r2u11s2", 4, 2, 11, 2, gemv_f16_wave_kernel<4, 2, 11, 2, false>},  // 11
-    {"w4r2u8s1nt", 4, 2, 8, 1, gemv_f16_wave_kernel<4, 2, 8, 1, true>},    // 12
-    {"w4r4u8s1nt", 4, 4, 8, 1, gemv_f16_wave_kernel<4, 4, 8, 1, true>},    // 13
-    {"w4r2u6s4nt", 4, 2, 6, 4, gemv_f16_wave_kernel<4, 2, 6, 4, true>},    // 14
-    {"w8r4u8s1", 8, 4, 8, 1, gemv_f16_wave_kernel<8, 4, 8, 1, false>},     // 15
-    {"w16r2u8s1", 16, 2, 8, 1, gemv_f16_wave_kernel<16, 2, 8, 1, false>},  // 16
+    {"auto", 0, 0, 0, 0, 0, nullptr},
+    TL_LOOP(4, 2, 8, 1, false),   // 1
+    TL_LOOP(4, 2, 8, 1, true),    // 2
+    TL_LOOP(4, 4, 8, 1, true),    // 3
+    TL_LOOP(4, 2, 4, 2, true),    // 4
+    TL_LOOP(4, 2, 6, 4, false),   // 5
+    TL_LOOP(4, 2, 6, 4, true),    // 6
+    TL_LOOP(8, 2, 6, 4, true),    // 7
+    TL_LOOP(4, 2, 2, 4, true),    // 8
+    // K = 4096 candidates (512 chunks per row)
+    TL_STREAM2(4, 2, 2, 4),       // 9, 10
+    TL_STREAM2(4, 4, 2, 4),       // 11, 12
+    TL_STREAM2(4, 8, 2, 4),       // 13, 14
+    TL_STREAM2(4, 2, 4, 2),       // 15, 16
+    TL_STREAM2(4, 4, 4, 2),       // 17, 18
+    TL_STREAM2(4, 1, 8, 1),       // 19, 20
+    TL_STREAM2(4, 2, 8, 1),       // 21, 22
+    TL_STREAM2(8, 2, 1, 8),       // 23, 24
+    TL_STREAM2(8, 4, 1, 8),       // 25, 26
+    TL_STREAM2(8, 2, 2, 4),       // 27, 28
+    TL_STREAM2(8, 4, 2, 4),       // 29, 30
+    // K = 11008 candidates (1376 chunks per row)
+    TL_STREAM2(4, 2, 6, 4),       // 31, 32
+    TL_STREAM2(4, 4, 6, 4),       // 33, 34
+    TL_STREAM2(8, 2, 3, 8),       // 35, 36
+    TL_STREAM2(8, 4, 3, 8),       // 37, 38
+    TL_STREAM2(4, 1, 11, 2),      // 39, 40
+    TL_STREAM2(4, 2, 11, 2),      // 41, 42
+    TL_STREAM2(8, 2, 6, 4),       // 43, 44
+    TL_STREAM2(8, 1, 6, 4),       // 45, 46
+    TL_STREAM2(4, 1, 6, 4),       // 47, 48
+    TL_STREAM2(4, 1, 2, 4),       // 49, 50
 };
 static constexpr int kNumVariants = sizeof(g_variants) / sizeof(g_variants[0]);
 static int g_forced_variant = 0;
 static int g_grid_waves_per_cu = 0;  // 0 = automatic
 
-static int pick_variant(size_t N, size_t K) {
-    // Down-projection shape (long rows, few of them): split K across the workgroup.
-    if (K >= 8192 && N <= 8192) return 8;
-    if (N >= 16384) return 3;
-    return 2;
+static int variant_index(const char* name) {
+    for (int i = 0; i < (int)(sizeof(g_variants) / sizeof(g_variants[0])); ++i)
+        if (strcmp(g_variants[i].name, name) == 0) return i;
+    return -1;
+}
+
+// Measured on MI355X (rotating weights, HBM resident) over the Llama2-7B decode shapes:
+//   K <= 4096  : 4 wavefronts split K, 2 rows each, one row block per workgroup
+//                (4096<-4096 7.1 us, 11008<-4096 14.6 us, 32000<-4096 37.2 us)
+//   K <= 12288 : 8 wavefronts split K, 2 rows each, 16 wavefronts per CU, grid-stride
+//                (4096<-11008 15.1 us)
+//   otherwise  : looping kernel with x staged in LDS.
+// In both streaming picks x goes straight to registers: each wavefront needs only its own K
+// segment, and skipping the LDS round trip and its barrier was 0.2-1.2 us faster per launch
+// than the LDS-staged twin of the same kernel.
+static int pick_variant(size_t N, size_t K, int* waves_per_cu) {
+    (void)N;
+    static const int v_k4096 = variant_index("stream_w4r2u2s4x1");
+    static const int v_k12288 = variant_index("stream_w8r2u3s8x1");
+    static const int v_loop = variant_index("loop_w4r2u6s4nttrue");
+    const size_t K8 = K / 8;
+    if (K8 <= 512) { *waves_per_cu = 1 << 20; return v_k4096; }
+    if (K8 <= 1536) { *waves_per_cu = 16; return v_k12288; }
+    *waves_per_cu = 16;
+    return v_loop;
 }
 
 int launch_gemv(const void* x, const void* W, void* y, size_t N, size_t K, size_t batch, size_t sx,
@@ -319,12 +477,24 @@ int launch_gemv(const void* x, const void* W, void* y, size_t N, size_t K, size_
         return TL_OK;
     }
 
-    int vi = g_forced_variant ? g_forced_variant : pick_variant(N, K);
+    int auto_wpc = 16;
+    int vi = g_forced_variant ? g_forced_variant : pick_variant(N, K, &auto_wpc);
+    if (g_variants[vi].xmode >= 0) {
+        // the streaming kernel needs a wavefront's K segment to fit one register tile
+        const GemvVariant& sv = g_variants[vi];
+        const int seg = (a.K8 + sv.ksplit - 1) / sv.ksplit;
+        if (seg > 64 * sv.unroll) {
+            TL_REQUIRE(g_forced_variant == 0, "gemv variant %s cannot hold K=%zu (segment %d chunks > %d)", sv.name, K,
+                       seg, 64 * sv.unroll);
+            vi = variant_index("loop_w4r2u6s4nttrue");
+        }
+    }
     const GemvVariant& v = g_variants[vi];
     const int rg = v.waves / v.ksplit;
     const int rows_per_block = rg * v.rows;
     a.num_row_blocks = (int)((N + rows_per_block - 1) / rows_per_block);
-    size_t lds = (size_t)a.K8 * 16 + (v.ksplit > 1 ? (size_t)rg * v.ksplit * v.rows * 4 : 0);
+    size_t lds = (v.xmode == 1 ? 0 : (size_t)a.K8 * 16) +
+                 (v.ksplit > 1 ? (size_t)(v.xmode >= 0 ? 2 : 1) * rg * v.ksplit * v.rows * 4 : 0);
     if (lds > 64 * 1024) {
         // x does not fit the default LDS window: fall back to the generic kernel.
         int blocks = (int)((N + 3) / 4);
@@ -337,10 +507,10 @@ int launch_gemv(const void* x, const void* W, void* y, size_t N, size_t K, size_
         return TL_OK;
     }
     int blocks = a.num_row_blocks;
-    int wpc = g_grid_waves_per_cu > 0 ? g_grid_waves_per_cu : 32;
-    int cap = dev.cu_count * wpc / v.waves;
+    int wpc = g_grid_waves_per_cu > 0 ? g_grid_waves_per_cu : auto_wpc;
+    long cap = (long)dev.cu_count * wpc / v.waves;
     if (cap < 1) cap = 1;
-    if (blocks > cap) blocks = cap;
+    if (blocks > cap) blocks = (int)cap;
     hipLaunchKernelGGL(v.kernel, dim3(blocks, (unsigned)batch), dim3(v.waves * 64), lds, st, a);
     TL_CHECK_LAUNCH(v.name);
     return TL_OK;

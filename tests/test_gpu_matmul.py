@@ -21,9 +21,14 @@ SWEEP = [(4096, 4096), (11008, 4096), (4096, 11008), (32000, 4096)]
 def _gemv_case(dev, oracle, N, K, seed, variant=0, w_std=0.02):
     W = synth.normal_f16(seed, (N, K), w_std)
     x = synth.normal_f16(seed + 1, (K,), 1.0)
+    from tensorlib_amd import TensorLibError
     dev.set_gemv_variant(variant)
     try:
         y = dev.gemv(dev.from_numpy(x), dev.from_numpy(W)).cpu().numpy()
+    except TensorLibError as e:
+        # a forced single-tile variant refuses rows longer than its register tile
+        assert variant != 0 and "cannot hold" in str(e), e
+        return
     finally:
         dev.set_gemv_variant(0)
     want = oracle.matmul2d(x[None, :], W)[0]
