@@ -41,6 +41,33 @@ def half_bits(x: float) -> int:
     return int(np.float16(x).view(np.uint16))
 
 
+def plan_matmul(a_shape, b_shape, out_shape=None):
+    """Shape logic of ``ops::matmul<dtype>::call2`` (tensorLib/src/ops/matmul.cpp:209-286) for
+    ``a[..., M, K] @ b[..., K, N]``: validates, right-aligns and broadcasts the batch dimensions.
+    Returns ``(a_batch, b_batch, out_batch, M, N, K)`` with the batch shapes padded to equal rank.
+    Raises ``ValueError`` where the reference throws ``std::invalid_argument``."""
+    a_shape, b_shape = list(a_shape), list(b_shape)
+    if len(a_shape) < 2 or len(b_shape) < 2:
+        raise ValueError("Tensors must have at least 2 dimensions for matmul.")
+    if a_shape[-1] != b_shape[-2]:
+        raise ValueError("Shape mismatch: the number of columns in the first tensor must match the number "
+                         "of rows in the second tensor.")
+    M, K = a_shape[-2:]
+    N = b_shape[-1]
+    ab, bb = a_shape[:-2], b_shape[:-2]
+    nb = max(len(ab), len(bb))
+    ab = [1] * (nb - len(ab)) + ab
+    bb = [1] * (nb - len(bb)) + bb
+    ob = []
+    for x, y in zip(ab, bb):
+        if x != y and x != 1 and y != 1:
+            raise ValueError("Shape mismatch: the batch dimensions must be broadcastable.")
+        ob.append(max(x, y))
+    if out_shape is not None and list(out_shape) != ob + [M, N]:
+        raise ValueError("result shape does not match new_shape")
+    return ab, bb, ob, M, N, K
+
+
 class HipDevice:
     """One GPU; all work goes to the library's stream (torch's current stream by default)."""
 
@@ -128,29 +155,12 @@ class HipDevice:
         boundary wants; for a Linear weight passed as ``W.t()`` no copy is made."""
         if a.device != b.device:
             raise ValueError("Tensors must be on the same device.")
-        if a.dim() < 2 or b.dim() < 2:
-            raise ValueError("Tensors must have at least 2 dimensions for matmul.")
-        if a.shape[-1] != b.shape[-2]:
-            raise ValueError("Shape mismatch: the number of columns in the first tensor must match the number "
-                             "of rows in the second tensor.")
+        ab, bb, obatch, M, N, K = plan_matmul(a.shape, b.shape, None if out is None else out.shape)
         A = a.contiguous()
         Bt = b.transpose(-2, -1).contiguous()  # [..., N, K]; a view of a Linear weight stays a view
-        M, K = A.shape[-2:]
-        N = Bt.shape[-2]
-        ab, bb = list(A.shape[:-2]), list(Bt.shape[:-2])
-        nb = max(len(ab), len(bb))
-        ab = [1] * (nb - len(ab)) + ab
-        bb = [1] * (nb - len(bb)) + bb
-        obatch = []
-        for x, y in zip(ab, bb):
-            if x != y and x != 1 and y != 1:
-                raise ValueError("Shape mismatch: the batch dimensions must be broadcastable.")
-            obatch.append(max(x, y))
         oshape = obatch + [M, N]
         if out is None:
             out = self.empty(*oshape)
-        elif list(out.shape) != oshape:
-            raise ValueError("result shape does not match new_shape")
         _req(out, name="out")
         batch = int(np.prod(obatch)) if obatch else 1
         if batch == 1:
