@@ -175,6 +175,18 @@ int tl_silu_mul_f16(void* out, const void* a, const void* b, size_t n);
 int tl_decode_attention_f16(void* out, const void* q, const void* cache_k, const void* cache_v,
                             int T, int n_heads, int head_dim);
 
+/* Decode-step glue after a fused q|k|v projection (qkv = [q | k | v], each n_heads*head_dim
+ * halves): rotary-embed q in place, rotary-embed k into cache_k[pos], copy v into cache_v[pos]
+ * (caches are [max_seq, n_heads, head_dim]).  Replaces two apply_rotary_emb launches and two
+ * setItem launches (model/llama2_7b/src/Transformer.cpp:47-53). */
+int tl_rope_qk_store_kv_f16(void* qkv, void* cache_k, void* cache_v, int pos, int n_heads, int head_dim);
+
+/* sum_out = a + b (one rounding) and norm_out = rmsnorm(sum_out) * weight per token: the
+ * residual EwiseAdd and the RMSNorm that follows it
+ * (model/llama2_7b/src/Transformer.cpp:167-171).  sum_out may alias a or b. */
+int tl_add_rms_norm_f16(void* sum_out, void* norm_out, const void* a, const void* b, const void* weight,
+                        float eps, int hidden_size, int num_tokens);
+
 /* mask[r,i,j] = (j > start_pos + i) ? -inf : 0 for r < reps, i < seqlen, j < start_pos+seqlen.
  * Replaces the element-by-element host loop of Transformer::get_mask
  * (model/llama2_7b/src/Transformer.cpp:231-261). */

@@ -155,6 +155,62 @@ causal_mask_kernel(half_t* mask, int seqlen, int start_pos, size_t n) {
     }
 }
 
+// Decode-step glue after the fused q|k|v GEMV: rotate q in place, rotate k and write it to
+// cache_k[pos], copy v to cache_v[pos].  One thread per (even, odd) pair of the 3*dim vector.
+__global__ void __launch_bounds__(256)
+rope_qk_store_kv_kernel(half_t* qkv, half_t* cache_k, half_t* cache_v, int pos, int n_heads, int head_dim) {
+    const int dim = n_heads * head_dim;
+    const int p = blockIdx.x * blockDim.x + threadIdx.x;  // pair index in [0, 3*dim/2)
+    if (p >= 3 * dim / 2) return;
+    const int which = p / (dim / 2);                       // 0 q, 1 k, 2 v
+    const int e = (p % (dim / 2)) * 2;                     // element index within the dim vector
+    half2_t v = *reinterpret_cast<const half2_t*>(qkv + which * dim + e);
+    if (which < 2) {
+        const int d = e % head_dim;
+        const float theta = (float)pos * 1.0f / powf(10000.0f, (float)d / (float)head_dim);
+        const float c = (float)(half_t)cosf(theta);
+        const float s = (float)(half_t)sinf(theta);
+        const float v0 = (float)v[0], v1 = (float)v[1];
+        v[0] = (half_t)(v0 * c - v1 * s);
+        v[1] = (half_t)(v0 * s + v1 * c);
+    }
+    if (which == 0)
+        *reinterpret_cast<half2_t*>(qkv + e) = v;
+    else if (which == 1)
+        *reinterpret_cast<half2_t*>(cache_k + (size_t)pos * dim + e) = v;
+    else
+        *reinterpret_cast<half2_t*>(cache_v + (size_t)pos * dim + e) = v;
+}
+
+// sum = a + b (one rounding, like the reference's EwiseAdd) and norm = rmsnorm(sum) * w in
+// one pass per token: the residual add of one sub-block and the RMSNorm that opens the next.
+__global__ void __launch_bounds__(256)
+add_rms_norm_kernel(half_t* sum_out, half_t* norm_out, const half_t* a, const half_t* b, const half_t* w, float eps,
+                    int hidden) {
+    __shared__ float red[4];
+    const size_t base = (size_t)blockIdx.x * hidden;
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+        const half_t s = (half_t)((float)a[base + i] + (float)b[base + i]);
+        sum_out[base + i] = s;
+        ss = __builtin_fmaf((float)s, (float)s, ss);
+    }
+    // wavefront then workgroup reduction
+    ss += dppf<0xB1>(ss);
+    ss += dppf<0x4E>(ss);
+    ss += dppf<0x141>(ss);
+    ss += dppf<0x140>(ss);
+    ss += __shfl_xor(ss, 16, 64);
+    ss += __shfl_xor(ss, 32, 64);
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = ss;
+    __syncthreads();
+    const float total = (red[0] + red[1]) + (red[2] + red[3]);
+    const float r = 1.0f / sqrtf(total / (float)hidden + eps);
+    // every thread re-reads the elements it wrote itself
+    for (int i = threadIdx.x; i < hidden; i += blockDim.x)
+        norm_out[base + i] = (half_t)((float)sum_out[base + i] * r * (float)w[i]);
+}
+
 // Library-owned fp32 workspace for the chunk partials, grown on demand.
 static std::mutex g_ws_mu;
 static float* g_ws = nullptr;
@@ -226,6 +282,33 @@ int tl_decode_attention_f16(void* out, const void* q, const void* cache_k, const
                            n_chunks);
         TL_CHECK_LAUNCH("decode_attn_merge_kernel");
     }
+    return TL_OK;
+}
+
+int tl_rope_qk_store_kv_f16(void* qkv, void* cache_k, void* cache_v, int pos, int n_heads, int head_dim) {
+    TL_ENSURE_INIT();
+    TL_REQUIRE(qkv && cache_k && cache_v, "tl_rope_qk_store_kv_f16: null pointer");
+    TL_REQUIRE(pos >= 0 && n_heads >= 1 && head_dim >= 2 && head_dim % 2 == 0,
+               "tl_rope_qk_store_kv_f16: bad sizes pos=%d n_heads=%d head_dim=%d", pos, n_heads, head_dim);
+    TL_REQUIRE(((uintptr_t)qkv & 3) == 0 && ((uintptr_t)cache_k & 3) == 0 && ((uintptr_t)cache_v & 3) == 0,
+               "tl_rope_qk_store_kv_f16: pointers must be 4-byte aligned");
+    const int pairs = 3 * n_heads * head_dim / 2;
+    hipLaunchKernelGGL(tl::rope_qk_store_kv_kernel, dim3((pairs + 255) / 256), dim3(256), 0, tl::stream(),
+                       (tl::half_t*)qkv, (tl::half_t*)cache_k, (tl::half_t*)cache_v, pos, n_heads, head_dim);
+    TL_CHECK_LAUNCH("rope_qk_store_kv_kernel");
+    return TL_OK;
+}
+
+int tl_add_rms_norm_f16(void* sum_out, void* norm_out, const void* a, const void* b, const void* weight, float eps,
+                        int hidden_size, int num_tokens) {
+    TL_ENSURE_INIT();
+    TL_REQUIRE(sum_out && norm_out && a && b && weight, "tl_add_rms_norm_f16: null pointer");
+    TL_REQUIRE(hidden_size > 0 && num_tokens >= 0, "tl_add_rms_norm_f16: bad sizes");
+    if (num_tokens == 0) return TL_OK;
+    hipLaunchKernelGGL(tl::add_rms_norm_kernel, dim3(num_tokens), dim3(256), 0, tl::stream(), (tl::half_t*)sum_out,
+                       (tl::half_t*)norm_out, (const tl::half_t*)a, (const tl::half_t*)b, (const tl::half_t*)weight,
+                       eps, hidden_size);
+    TL_CHECK_LAUNCH("add_rms_norm_kernel");
     return TL_OK;
 }
 

@@ -1,0 +1,369 @@
+// Host-side Llama2 driver: the caller of the matmul hot path.
+//
+// Issues, through the Device-shaped backend (include/tl_hip_device.hpp), the op sequence of the
+// reference's model code:
+//   Attention::forward        model/llama2_7b/src/Transformer.cpp:26-112
+//   FeedForward::forward      model/llama2_7b/src/Transformer.cpp:132-145
+//   TransformerBlock::forward model/llama2_7b/src/Transformer.cpp:160-178
+//   Transformer::forward      model/llama2_7b/src/Transformer.cpp:263-299
+//   Llama2::generate          model/llama2_7b/src/llama2.cpp:15-101
+// with the intended dataflow x_norm <- rmsnorm(x) (what the reference's GPU path executes).
+// Buffers are allocated once, like ActivationBuffer (model/llama2_7b/include/ActivationBuffer.hpp:10-36),
+// but score/mask scratch is sized by max_tokens * max_seq_len instead of max_seq_len^2.
+#include <chrono>
+#include <cmath>
+#include <cstdarg>
+#include <cstdio>
+#include <memory>
+#include <stdexcept>
+#include <string>
+#include <vector>
+
+#include "tensorlib_amd.h"
+#include "tensorlib_llama2.h"
+#include "tl_hip_device.hpp"
+
+namespace {
+
+using half = tl::half;
+using Dev = HIP<half>;
+
+thread_local char g_err[512] = {0};
+
+int fail(const char* fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+    return -1;
+}
+
+void ck(int status, const char* what) { tl::throw_on_error(status, what); }
+
+// A device buffer plus the Device-shaped object that adopts it (non-owning).
+struct Buf {
+    half* p = nullptr;
+    size_t n = 0;
+    std::unique_ptr<Dev> dev;
+    void alloc(size_t elems) {
+        void* q = nullptr;
+        ck(tl_malloc(&q, elems * sizeof(half)), "tl_malloc");
+        p = static_cast<half*>(q);
+        n = elems;
+        dev.reset(new Dev(elems, p));
+    }
+    void release() {
+        dev.reset();
+        if (p) tl_free(p);
+        p = nullptr;
+    }
+};
+
+struct LayerWeights {
+    const half *att_norm = nullptr, *wq = nullptr, *wk = nullptr, *wv = nullptr, *wo = nullptr;
+    const half *ffn_norm = nullptr, *w1 = nullptr, *w2 = nullptr, *w3 = nullptr;
+};
+
+}  // namespace
+
+struct tlm_model {
+    int dim, hidden, n_layers, n_heads, head_dim, vocab, max_seq, max_tokens;
+    float eps;
+    const half* tok_emb = nullptr;
+    const half* final_norm = nullptr;
+    const half* classifier = nullptr;
+    std::vector<LayerWeights> layers;
+    std::vector<Buf> cache_k, cache_v;  // per layer [max_seq, n_heads, head_dim]
+    Buf x, x_norm, x_residual, qkv, x13, x2, scores, scores2, mask, xq_c, keys_c, values_c, s_v, o_c, logits;
+    int* d_tokens = nullptr;   // [max_tokens + generated]
+    int d_tokens_cap = 0;
+    Dev scratch_dev;           // method holder for calls that take explicit pointers
+
+    half* xq(int) { return qkv.p; }
+    half* xk(int S) { return qkv.p + (size_t)S * dim; }
+    half* xv(int S) { return qkv.p + (size_t)2 * S * dim; }
+    half* x1(int) { return x13.p; }
+    half* x3(int S) { return x13.p + (size_t)S * hidden; }
+
+    void check_weights() const {
+        if (!tok_emb || !final_norm || !classifier) throw std::runtime_error("embedding/final norm/classifier not set");
+        for (int l = 0; l < n_layers; ++l) {
+            const LayerWeights& w = layers[l];
+            if (!w.att_norm || !w.wq || !w.wk || !w.wv || !w.wo || !w.ffn_norm || !w.w1 || !w.w2 || !w.w3)
+                throw std::runtime_error("weights of layer " + std::to_string(l) + " not set");
+        }
+    }
+
+    void matmul2d(const half* A, const half* B, half* C, size_t M, size_t N, size_t K) {
+        scratch_dev.matmul2d(A, B, C, M, N, K);
+    }
+
+    // ---- the reference's op list, one call per op -------------------------------------------
+    void block_chain(int l, int S, int start_pos, bool use_mask) {
+        const LayerWeights& w = layers[l];
+        const int T = start_pos + S, H = n_heads, D = head_dim;
+        const size_t sd = (size_t)S * dim;
+        // attention_norm.forward(x -> x_norm)                              Transformer.cpp:165
+        scratch_dev.rms_norm(x_norm.p, x.p, const_cast<half*>(w.att_norm), eps, dim, S);
+        // wq / wk / wv .forward                                            Transformer.cpp:35-37
+        matmul2d(x_norm.p, w.wq, xq(S), S, dim, dim);
+        matmul2d(x_norm.p, w.wk, xk(S), S, dim, dim);
+        matmul2d(x_norm.p, w.wv, xv(S), S, dim, dim);
+        // apply_rotary_emb in place                                         Transformer.cpp:47-48
+        scratch_dev.apply_rotary_emb(xq(S), xq(S), start_pos, 1, S, H, D);
+        scratch_dev.apply_rotary_emb(xk(S), xk(S), start_pos, 1, S, H, D);
+        // cache_k/v.setItem({0,bsz},{start_pos,start_pos+seqlen})            Transformer.cpp:51-53
+        const std::vector<int> shp_new = {1, S, H, D};
+        const std::vector<int> str_cache = {max_seq * dim, dim, D, 1};
+        cache_k[l].dev->setItemEwise(xk(S), shp_new, str_cache, (size_t)start_pos * dim, sd);
+        cache_v[l].dev->setItemEwise(xv(S), shp_new, str_cache, (size_t)start_pos * dim, sd);
+        // xq.transpose(1,2).contiguous(xq_c)                                Transformer.cpp:60
+        {
+            Dev q(sd, xq(S));
+            q.contiguous(xq_c.p, {1, H, S, D}, {S * dim, D, dim, 1}, 0, sd);
+        }
+        // keys -> [1,H,T,D] contiguous, values -> [1,H,D,T] contiguous      Transformer.cpp:61-80
+        cache_k[l].dev->contiguous(keys_c.p, {1, H, T, D}, {max_seq * dim, D, dim, 1}, 0, (size_t)T * dim);
+        cache_v[l].dev->contiguous(values_c.p, {1, H, D, T}, {max_seq * dim, D, 1, dim}, 0, (size_t)T * dim);
+        // xq.matmul(keys): n_heads matmul2d calls in the reference          Transformer.cpp:92, matmul.cpp:297-321
+        ck(tl_matmul2d_batched_f16(xq_c.p, keys_c.p, scores.p, S, T, D, H, (size_t)S * D, (size_t)T * D, (size_t)S * T),
+           "scores");
+        const size_t ns = (size_t)H * S * T;
+        // ScalarDiv(sqrt(head_dim))                                          Transformer.cpp:94
+        scores.dev->div(scores.p, (half)std::sqrt((float)D), ns);
+        // EwiseAdd(mask)                                                     Transformer.cpp:99-102
+        if (use_mask) scores.dev->add(scores.p, mask.p, ns);
+        // softmax(3)                                                         Transformer.cpp:105
+        scores.dev->softmax(scores2.p, (size_t)H * S, T);
+        // scores.matmul(values)                                              Transformer.cpp:107
+        ck(tl_matmul2d_batched_f16(scores2.p, values_c.p, s_v.p, S, D, T, H, (size_t)S * T, (size_t)D * T, (size_t)S * D),
+           "scores.values");
+        // output.transpose(1,2).contiguous(o_c)                             Transformer.cpp:109
+        s_v.dev->contiguous(o_c.p, {1, S, H, D}, {H * S * D, D, S * D, 1}, 0, sd);
+        // wo.forward(output -> x_norm)                                      Transformer.cpp:111
+        matmul2d(o_c.p, w.wo, x_norm.p, S, dim, dim);
+        // h = x + attention                                                  Transformer.cpp:169
+        x.dev->add(x_residual.p, x_norm.p, sd);
+        // ffn_norm.forward(h -> x_norm)                                      Transformer.cpp:171
+        scratch_dev.rms_norm(x_norm.p, x_residual.p, const_cast<half*>(w.ffn_norm), eps, dim, S);
+        // FeedForward::forward                                               Transformer.cpp:132-145
+        const size_t sh = (size_t)S * hidden;
+        matmul2d(x_norm.p, w.w1, x1(S), S, hidden, dim);
+        {
+            Dev d1(sh, x1(S));
+            d1.silu(x1(S), sh);
+            matmul2d(x_norm.p, w.w3, x3(S), S, hidden, dim);
+            d1.mul(x2.p, x3(S), sh);
+        }
+        matmul2d(x2.p, w.w2, x.p, S, dim, hidden);
+        // out = h + ffn ; activation_buffer.x.setItem(h)                     Transformer.cpp:175, 291
+        x_residual.dev->add(x_residual.p, x.p, sd);
+        x.dev->setItemEwise(x_residual.p, {1, S, dim}, {S * dim, dim, 1}, 0, sd);
+    }
+
+    // ---- fused single-token step --------------------------------------------------------------
+    void gemv(const half* xin, const half* W, half* y, size_t N, size_t K) { ck(tl_gemv_f16(xin, W, y, N, K), "gemv"); }
+
+    void decode_fused(int pos) {
+        const int H = n_heads, D = head_dim;
+        ck(tl_rms_norm_f16(x_norm.p, x.p, layers[0].att_norm, eps, dim, 1), "rms_norm");
+        for (int l = 0; l < n_layers; ++l) {
+            const LayerWeights& w = layers[l];
+            const size_t dd = (size_t)dim * dim;
+            if (w.wk == w.wq + dd && w.wv == w.wk + dd) {
+                gemv(x_norm.p, w.wq, qkv.p, (size_t)3 * dim, dim);
+            } else {
+                gemv(x_norm.p, w.wq, xq(1), dim, dim);
+                gemv(x_norm.p, w.wk, xk(1), dim, dim);
+                gemv(x_norm.p, w.wv, xv(1), dim, dim);
+            }
+            ck(tl_rope_qk_store_kv_f16(qkv.p, cache_k[l].p, cache_v[l].p, pos, H, D), "rope_qk_store_kv");
+            ck(tl_decode_attention_f16(o_c.p, qkv.p, cache_k[l].p, cache_v[l].p, pos + 1, H, D), "decode_attention");
+            gemv(o_c.p, w.wo, x_norm.p, dim, dim);
+            // h = x + attn ; x_norm = rmsnorm(h) * ffn_norm
+            ck(tl_add_rms_norm_f16(x_residual.p, x_norm.p, x.p, x_norm.p, w.ffn_norm, eps, dim, 1), "add_rms_norm");
+            if (w.w3 == w.w1 + (size_t)hidden * dim) {
+                gemv(x_norm.p, w.w1, x13.p, (size_t)2 * hidden, dim);
+            } else {
+                gemv(x_norm.p, w.w1, x1(1), hidden, dim);
+                gemv(x_norm.p, w.w3, x3(1), hidden, dim);
+            }
+            ck(tl_silu_mul_f16(x2.p, x1(1), x3(1), hidden), "silu_mul");
+            gemv(x2.p, w.w2, x.p, dim, hidden);
+            // x = h + ffn ; x_norm = rmsnorm(x) * (next layer's attention norm | final norm)
+            const half* next_norm = (l + 1 < n_layers) ? layers[l + 1].att_norm : final_norm;
+            ck(tl_add_rms_norm_f16(x.p, x_norm.p, x_residual.p, x.p, next_norm, eps, dim, 1), "add_rms_norm");
+        }
+    }
+
+    half* forward(const int* dev_tokens, int S, int start_pos, int mode, bool all_logits) {
+        check_weights();
+        if (S < 1 || S > max_tokens) throw std::runtime_error("n_tokens out of range [1, max_tokens]");
+        if (start_pos < 0 || start_pos + S > max_seq) throw std::runtime_error("positions exceed max_seq_len");
+        // tok_embeddings.forward                                             Transformer.cpp:274
+        ck(tl_embedding_f16(x.p, tok_emb, dev_tokens, S, dim, vocab), "embedding");
+        if (mode == TLM_MODE_FUSED && S == 1) {
+            decode_fused(start_pos);   // leaves rmsnorm(x) * final_norm in x_norm
+            gemv(x_norm.p, classifier, logits.p, vocab, dim);
+            return logits.p;
+        }
+        const bool use_mask = S > 1;   // get_mask: nullopt when seqlen <= 1   Transformer.cpp:234
+        if (use_mask) ck(tl_causal_mask_f16(mask.p, n_heads, S, start_pos), "causal_mask");
+        for (int l = 0; l < n_layers; ++l) block_chain(l, S, start_pos, use_mask);
+        // norm.forward ; output.forward                                      Transformer.cpp:295-296
+        if (all_logits) {
+            scratch_dev.rms_norm(x_norm.p, x.p, const_cast<half*>(final_norm), eps, dim, S);
+            matmul2d(x_norm.p, classifier, logits.p, S, vocab, dim);
+        } else {
+            // only the last position's logits are consumed (llama2.cpp:53-57)
+            scratch_dev.rms_norm(x_norm.p, x.p + (size_t)(S - 1) * dim, const_cast<half*>(final_norm), eps, dim, 1);
+            matmul2d(x_norm.p, classifier, logits.p, 1, vocab, dim);
+        }
+        return logits.p;
+    }
+};
+
+extern "C" {
+
+const char* tlm_last_error(void) { return g_err; }
+
+int tlm_create(tlm_model** out, int dim, int hidden_dim, int n_layers, int n_heads, int vocab_size, int max_seq_len,
+               float norm_eps, int max_tokens) {
+    if (!out) return fail("tlm_create: out is null");
+    *out = nullptr;
+    if (dim <= 0 || hidden_dim <= 0 || n_layers <= 0 || n_heads <= 0 || vocab_size <= 0 || max_seq_len <= 0 ||
+        max_tokens <= 0 || dim % n_heads != 0 || (dim / n_heads) % 2 != 0 || max_tokens > max_seq_len)
+        return fail("tlm_create: bad configuration");
+    std::unique_ptr<tlm_model> m(new tlm_model());
+    try {
+        m->dim = dim; m->hidden = hidden_dim; m->n_layers = n_layers; m->n_heads = n_heads;
+        m->head_dim = dim / n_heads; m->vocab = vocab_size; m->max_seq = max_seq_len; m->max_tokens = max_tokens;
+        m->eps = norm_eps;
+        m->layers.resize(n_layers);
+        m->cache_k.resize(n_layers);
+        m->cache_v.resize(n_layers);
+        const size_t S = max_tokens, sd = S * dim;
+        for (int l = 0; l < n_layers; ++l) {
+            m->cache_k[l].alloc((size_t)max_seq_len * dim);
+            m->cache_v[l].alloc((size_t)max_seq_len * dim);
+        }
+        m->x.alloc(sd); m->x_norm.alloc(sd); m->x_residual.alloc(sd);
+        m->qkv.alloc(3 * sd);
+        m->x13.alloc(2 * S * hidden_dim);
+        m->x2.alloc(S * hidden_dim);
+        const size_t sc = (size_t)n_heads * S * max_seq_len;
+        m->scores.alloc(sc); m->scores2.alloc(sc); m->mask.alloc(sc);
+        m->xq_c.alloc(sd); m->s_v.alloc(sd); m->o_c.alloc(sd);
+        m->keys_c.alloc((size_t)max_seq_len * dim);
+        m->values_c.alloc((size_t)max_seq_len * dim);
+        m->logits.alloc(S * vocab_size);
+        m->d_tokens_cap = max_seq_len + 8;
+        void* p = nullptr;
+        ck(tl_malloc(&p, (size_t)m->d_tokens_cap * sizeof(int)), "tl_malloc tokens");
+        m->d_tokens = static_cast<int*>(p);
+    } catch (const std::exception& e) {
+        return fail("tlm_create: %s", e.what());
+    }
+    *out = m.release();
+    return 0;
+}
+
+int tlm_destroy(tlm_model* m) {
+    if (!m) return 0;
+    tl_synchronize();
+    for (auto& b : m->cache_k) b.release();
+    for (auto& b : m->cache_v) b.release();
+    for (Buf* b : {&m->x, &m->x_norm, &m->x_residual, &m->qkv, &m->x13, &m->x2, &m->scores, &m->scores2, &m->mask,
+                   &m->xq_c, &m->keys_c, &m->values_c, &m->s_v, &m->o_c, &m->logits})
+        b->release();
+    if (m->d_tokens) tl_free(m->d_tokens);
+    delete m;
+    return 0;
+}
+
+int tlm_set_weight(tlm_model* m, int kind, int layer, const void* dev_ptr) {
+    if (!m || !dev_ptr) return fail("tlm_set_weight: null argument");
+    const half* p = static_cast<const half*>(dev_ptr);
+    const bool per_layer = kind >= TLM_W_ATT_NORM && kind <= TLM_W_W3;
+    if (per_layer && (layer < 0 || layer >= m->n_layers)) return fail("tlm_set_weight: layer %d out of range", layer);
+    switch (kind) {
+        case TLM_W_TOK_EMB: m->tok_emb = p; break;
+        case TLM_W_ATT_NORM: m->layers[layer].att_norm = p; break;
+        case TLM_W_WQ: m->layers[layer].wq = p; break;
+        case TLM_W_WK: m->layers[layer].wk = p; break;
+        case TLM_W_WV: m->layers[layer].wv = p; break;
+        case TLM_W_WO: m->layers[layer].wo = p; break;
+        case TLM_W_FFN_NORM: m->layers[layer].ffn_norm = p; break;
+        case TLM_W_W1: m->layers[layer].w1 = p; break;
+        case TLM_W_W2: m->layers[layer].w2 = p; break;
+        case TLM_W_W3: m->layers[layer].w3 = p; break;
+        case TLM_W_FINAL_NORM: m->final_norm = p; break;
+        case TLM_W_CLASSIFIER: m->classifier = p; break;
+        default: return fail("tlm_set_weight: unknown kind %d", kind);
+    }
+    return 0;
+}
+
+int tlm_forward(tlm_model* m, const int* dev_tokens, int n_tokens, int start_pos, int mode, int all_logits,
+                void** logits_out) {
+    if (!m || !dev_tokens) return fail("tlm_forward: null argument");
+    if (mode != TLM_MODE_REFERENCE_CHAIN && mode != TLM_MODE_FUSED) return fail("tlm_forward: unknown mode %d", mode);
+    try {
+        half* lg = m->forward(dev_tokens, n_tokens, start_pos, mode, all_logits != 0);
+        if (logits_out) *logits_out = lg;
+    } catch (const std::exception& e) {
+        return fail("tlm_forward: %s", e.what());
+    }
+    return 0;
+}
+
+int tlm_generate(tlm_model* m, const int* host_prompt, int n_prompt, int n_generate, int mode, int* host_out_tokens,
+                 double* prefill_seconds, double* decode_seconds) {
+    if (!m || !host_prompt || !host_out_tokens) return fail("tlm_generate: null argument");
+    if (n_prompt < 1 || n_prompt > m->max_tokens) return fail("tlm_generate: prompt length %d not in [1,%d]", n_prompt, m->max_tokens);
+    if (n_generate < 1 || n_prompt + n_generate > m->max_seq) return fail("tlm_generate: sequence exceeds max_seq_len");
+    if (n_prompt + n_generate > m->d_tokens_cap) return fail("tlm_generate: token buffer too small");
+    using clock = std::chrono::steady_clock;
+    try {
+        // prompt ids and generated ids live in one device array: d_tokens[i] is the token at position i
+        ck(tl_memcpy_h2d(m->d_tokens, host_prompt, (size_t)n_prompt * sizeof(int)), "prompt h2d");
+        ck(tl_synchronize(), "sync");
+        auto t0 = clock::now();
+        half* lg = m->forward(m->d_tokens, n_prompt, 0, mode, false);
+        ck(tl_argmax_f16(m->d_tokens + n_prompt, lg, m->vocab, m->vocab), "argmax");
+        ck(tl_synchronize(), "sync");
+        auto t1 = clock::now();
+        // greedy loop (llama2.cpp:81-95) without the per-step host read of the token: the id stays
+        // on the device and feeds the next embedding lookup directly
+        for (int i = 1; i < n_generate; ++i) {
+            const int pos = n_prompt + i - 1;
+            lg = m->forward(m->d_tokens + pos, 1, pos, mode, false);
+            ck(tl_argmax_f16(m->d_tokens + pos + 1, lg, m->vocab, m->vocab), "argmax");
+        }
+        ck(tl_synchronize(), "sync");
+        auto t2 = clock::now();
+        ck(tl_memcpy_d2h(host_out_tokens, m->d_tokens + n_prompt, (size_t)n_generate * sizeof(int)), "tokens d2h");
+        if (prefill_seconds) *prefill_seconds = std::chrono::duration<double>(t1 - t0).count();
+        if (decode_seconds) *decode_seconds = std::chrono::duration<double>(t2 - t1).count();
+    } catch (const std::exception& e) {
+        return fail("tlm_generate: %s", e.what());
+    }
+    return 0;
+}
+
+int tlm_get_buffer(tlm_model* m, int which, int layer, void** dev_ptr) {
+    if (!m || !dev_ptr) return fail("tlm_get_buffer: null argument");
+    switch (which) {
+        case TLM_BUF_X: *dev_ptr = m->x.p; return 0;
+        case TLM_BUF_LOGITS: *dev_ptr = m->logits.p; return 0;
+        case TLM_BUF_NEXT_TOKEN: *dev_ptr = m->d_tokens; return 0;
+        case TLM_BUF_CACHE_K:
+        case TLM_BUF_CACHE_V:
+            if (layer < 0 || layer >= m->n_layers) return fail("tlm_get_buffer: layer %d out of range", layer);
+            *dev_ptr = which == TLM_BUF_CACHE_K ? m->cache_k[layer].p : m->cache_v[layer].p;
+            return 0;
+        default: return fail("tlm_get_buffer: unknown buffer %d", which);
+    }
+}
+
+}  // extern "C"

@@ -46,3 +46,14 @@ def assert_close_f16(got, want, rtol=1e-2, atol=1e-3, what=""):
         raise AssertionError(
             f"{what}: {int(bad.sum())}/{bad.size} elements outside atol={atol} rtol={rtol}; first at {tuple(idx)}: "
             f"got {g[tuple(idx)]} want {w[tuple(idx)]}; max abs err {np.nanmax(np.where(bad, err, 0))}")
+
+
+def assert_close_scaled(got, want, rtol=1e-2, scale_tol=1e-2, what=""):
+    """Gate for op CHAINS (a transformer block, the whole model): every one of the ~25 ops of a block
+    rounds to fp16, and two correct fp32-accumulating implementations differ by a rounding step
+    after each of them, so the absolute slack is tied to the tensor's own scale:
+    |got - want| <= rtol*|want| + scale_tol*rms(want)."""
+    import numpy as np
+    w = np.asarray(want, dtype=np.float32)
+    rms = float(np.sqrt(np.mean(np.square(w[np.isfinite(w)])))) if w.size else 0.0
+    assert_close_f16(got, want, rtol, scale_tol * rms, what + f" (rms {rms:.3g})")

@@ -27,6 +27,18 @@ def test_binding_covers_the_header_exactly():
     assert sorted(_lib._PROTOS) == _lib.declared_symbols()
 
 
+def test_llama2_driver_exports_its_header():
+    import re as _re
+    from tensorlib_amd import llama2
+    text = open(os.path.join(ROOT, "include", "tensorlib_llama2.h")).read()
+    text = _re.sub(r"/\*.*?\*/", "", text, flags=_re.S)
+    declared = sorted(set(_re.findall(r"\b(tlm_[a-z0-9_]+)\s*\(", text)))
+    assert sorted(llama2._PROTOS) == declared
+    ctypes.CDLL(_lib.LIB_PATH, mode=ctypes.RTLD_GLOBAL)
+    handle = ctypes.CDLL(llama2.LLAMA2_LIB_PATH)
+    assert not [s for s in declared if not hasattr(handle, s)]
+
+
 def test_header_cites_the_reference_for_each_hot_path_entry():
     text = open(_lib.HEADER).read()
     for sym in ["tl_matmul2d_f16", "tl_gemv_f16", "tl_hgemm_f16", "tl_rms_norm_f16", "tl_apply_rotary_emb_f16",
