@@ -37,8 +37,8 @@ HGEMM_SHAPES = [(2048, 4096, 4096), (2048, 11008, 4096), (2048, 32000, 4096), (2
 
 # HBM bytes per GEMV launch measured with rocprofv3 --pmc (FETCH_SIZE, WRITE_SIZE), averaged over
 # the four sweep launches and scaled by the same counters' reading for a copy kernel of known
-# size; None until the counter profile under profiles/ exists.
-GEMV_TRAFFIC_BYTES_PER_LAUNCH = None
+# size (FETCH_SIZE x 1.9997 KiB, WRITE_SIZE x 1.0000 KiB); algorithmic bytes per launch are 119,050,624.
+GEMV_TRAFFIC_BYTES_PER_LAUNCH = 119_422_121  # profiles/gemv_decode_sweep_hbm_traffic.txt
 
 
 def parse_args():
@@ -48,6 +48,9 @@ def parse_args():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-extra", action="store_true", help="skip the HGEMM / per-shape / model extras")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also launch plain 256 MiB copies (strided_copy_kernel) so that a rocprofv3 --pmc run "
+                         "of this command holds a kernel of known HBM traffic next to the GEMV")
     return ap.parse_args()
 
 
@@ -130,6 +133,14 @@ def main():
         for W, x, y in s:
             dev.matmul2d(x, W, y)
 
+    if args.copy_calibration:
+        src = torch.zeros(1 << 27, device="cuda", dtype=torch.float16)   # 256 MiB read + 256 MiB written
+        dst = torch.empty_like(src)
+        for _ in range(5):
+            dev.contiguous(src, (1 << 27,), (1,), 0, out=dst)
+        torch.cuda.synchronize()
+        del src, dst
+
     for _ in range(args.warmup):
         step()
     wall, ev = time_region(step, args.steps, torch)
@@ -163,7 +174,7 @@ def main():
             "unit": "GB/s",
             "frac": round(achieved / HBM_PEAK_GBS, 4),
             "traffic": GEMV_TRAFFIC_BYTES_PER_LAUNCH,
-            "kernel": "gemv_f16_wave_kernel",
+            "kernel": "gemv_f16_stream_kernel",
             "bytes_per_launch": step_bytes / len(SWEEP),
             "avg_launch_us": round(avg_launch_s * 1e6, 3),
         },
