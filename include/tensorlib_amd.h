@@ -106,6 +106,8 @@ int tl_set_gemv_variant(int variant);
 int tl_set_hgemm_variant(int variant);
 const char* tl_gemv_variant_name(int variant);
 const char* tl_hgemm_variant_name(int variant);
+/* Tuning hook: force the number of K splits of the MFMA GEMM (0 = automatic). */
+int tl_set_hgemm_splits(int splits);
 /* Tuning hook: cap the GEMV grid at `waves` resident wavefronts per compute unit (0 = default). */
 int tl_set_gemv_grid_waves_per_cu(int waves);
 

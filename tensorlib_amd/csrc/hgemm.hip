@@ -15,6 +15,9 @@
 // 32 rows a ds_read_b128 touches fall in distinct bank groups), double buffered: while the
 // MFMAs of step k run out of one buffer, the global loads of step k+1 are in flight in
 // registers and are written to the other buffer before the single barrier of the step.
+#include <cstring>
+#include <mutex>
+
 #include "tl_internal.h"
 
 namespace tl {
@@ -26,6 +29,10 @@ struct HgemmArgs {
     int M, N, K;
     int tiles_m, tiles_n;
     long sa, sb, sc;  // batch strides in elements
+    // split-K (direct-to-LDS kernel only): blockIdx.z walks K tiles [z*kt_per_split, ...) and writes
+    // fp32 partial sums to partial[z][M][N]; a second kernel adds the splits in order.
+    int kt_per_split;
+    float* partial;
 };
 
 constexpr int kPad = 8;  // halves of padding per LDS row
@@ -175,6 +182,244 @@ __global__ void __launch_bounds__(WM* WN * 64) hgemm_f16_mfma_kernel(HgemmArgs a
     }
 }
 
+// ------------------------------------------------------------------------------------------
+// Direct-to-LDS variant.  Tiles go HBM -> LDS with global_load_lds_dwordx4 (no VGPR staging,
+// no ds_write), through a ring of STAGES LDS buffers, so the loads of tile k+STAGES-1 are in
+// flight while tile k feeds the MFMAs.  A wavefront-load writes 1 KiB of LDS in lane order, so
+// the bank-conflict-free layout is obtained by permuting WHICH 16-byte chunk of a row each lane
+// fetches: the chunk stored at slot p of tile row r is chunk p ^ ((r / RPL) % CPR), where RPL
+// rows fill one 256-byte LDS line and CPR is the number of chunks per row.  The 16 rows a
+// ds_read_b128 group touches then land in 16 different 16-byte bank groups.
+// Requirements: K % BK == 0 (no zero fill is possible on this path), K % 8 == 0, aligned operands.
+template <int N_>
+__device__ __forceinline__ void wait_vmcnt_and_barrier() {
+    // waits until at most N_ of this wavefront's global->LDS loads are outstanding and all of its
+    // LDS reads have returned, then joins the workgroup barrier; the "memory" clobber keeps LDS
+    // accesses on their side of it
+    asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(N_) : "memory");
+}
+
+template <int BM, int BN, int BK, int WM, int WN, int STAGES, bool PIPE>
+__global__ void __launch_bounds__(WM* WN * 64) hgemm_f16_dlds_kernel(HgemmArgs a) {
+    constexpr int NW = WM * WN;
+    constexpr int RB = BK * 2;                 // bytes per tile row
+    constexpr int CPR = BK / 8;                // 16-byte chunks per tile row
+    constexpr int RPL = 256 / RB;              // tile rows per 256-byte LDS line
+    constexpr int RPW = 1024 / RB;             // tile rows written by one wavefront-load
+    constexpr int A_LOADS = BM / RPW / NW;     // wavefront-loads per stage, per wavefront
+    constexpr int B_LOADS = BN / RPW / NW;
+    constexpr int LPW = A_LOADS + B_LOADS;
+    constexpr int A_BYTES = BM * RB;
+    constexpr int STAGE_BYTES = (BM + BN) * RB;
+    constexpr int TM = BM / WM, TN = BN / WN;
+    constexpr int MT = TM / 32, NT = TN / 32;
+    constexpr int KS = BK / 16;
+    static_assert(BK == 32 || BK == 64, "BK must be 32 or 64");
+    static_assert(BM % (RPW * NW) == 0 && BN % (RPW * NW) == 0, "tile rows must split over the wavefronts");
+    static_assert(STAGES >= 2 && STAGES <= 4 && LPW * (STAGES - 2) < 64, "vmcnt is a 6-bit counter");
+
+    extern __shared__ __attribute__((aligned(1024))) unsigned char smem_raw[];
+    typedef __attribute__((address_space(3))) unsigned char lds_byte_t;
+    lds_byte_t* lds = (lds_byte_t*)smem_raw;
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave / WN, wn = wave % WN;
+
+    int tile_m, tile_n;
+    tile_of_block(blockIdx.x, gridDim.x, a.tiles_m, tile_m, tile_n);
+    const int m0 = tile_m * BM, n0 = tile_n * BN;
+    const int batch = blockIdx.y;
+    const half_t* __restrict__ A = a.A + (size_t)batch * a.sa;
+    const half_t* __restrict__ B = a.B + (size_t)batch * a.sb;
+    half_t* __restrict__ C = a.C + (size_t)batch * a.sc;
+    const int M = a.M, N = a.N, K = a.K;
+
+    // ---- loader: wavefront-load j of this wavefront covers tile rows (j*NW + wave)*RPW .. +RPW ----
+    const int ld_row_in_group = lane / CPR;
+    const int ld_slot = lane % CPR;
+    const half_t* a_src[A_LOADS];
+    const half_t* b_src[B_LOADS];
+#pragma unroll
+    for (int j = 0; j < A_LOADS; ++j) {
+        const int r = (j * NW + wave) * RPW + ld_row_in_group;  // tile row
+        const int c = ld_slot ^ ((r / RPL) % CPR);              // chunk of that row this lane fetches
+        int gr = m0 + r;
+        gr = gr < M ? gr : M - 1;
+        a_src[j] = A + (size_t)gr * K + c * 8;
+    }
+#pragma unroll
+    for (int j = 0; j < B_LOADS; ++j) {
+        const int r = (j * NW + wave) * RPW + ld_row_in_group;
+        const int c = ld_slot ^ ((r / RPL) % CPR);
+        int gr = n0 + r;
+        gr = gr < N ? gr : N - 1;
+        b_src[j] = B + (size_t)gr * K + c * 8;
+    }
+    auto issue_loads = [&](int stage, int kt) {
+#if defined(TL_EXP_NOLOAD)
+        if (kt >= STAGES) return;
+#endif
+        lds_byte_t* sa = lds + stage * STAGE_BYTES;
+        lds_byte_t* sb = sa + A_BYTES;
+        const size_t koff = (size_t)kt * BK;
+#pragma unroll
+        for (int j = 0; j < A_LOADS; ++j)
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(a_src[j] + koff),
+                                             (__attribute__((address_space(3))) void*)(sa + (j * NW + wave) * 1024), 16,
+                                             0, 0);
+#pragma unroll
+        for (int j = 0; j < B_LOADS; ++j)
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(b_src[j] + koff),
+                                             (__attribute__((address_space(3))) void*)(sb + (j * NW + wave) * 1024), 16,
+                                             0, 0);
+    };
+
+    // ---- fragment reader: row (lane % 32) of a 32-row MFMA tile, chunk 2*ks + lane/32 ----
+    const int fr_row = lane & 31;
+    const int fr_sw = (fr_row / RPL) % CPR;
+    int fr_off[KS];
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) fr_off[ks] = fr_row * RB + (((ks * 2 + (lane >> 5)) ^ fr_sw) * 16);
+    const int a_base = wm * TM * RB;
+    const int b_base = A_BYTES + wn * TN * RB;
+
+    float16_t acc[MT][NT];
+#pragma unroll
+    for (int i = 0; i < MT; ++i)
+#pragma unroll
+        for (int j = 0; j < NT; ++j)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+
+    const int KT_all = K / BK;
+    const int kt_begin = (int)blockIdx.z * a.kt_per_split;
+    const int KT = (KT_all - kt_begin) < a.kt_per_split ? (KT_all - kt_begin) : a.kt_per_split;
+#pragma unroll
+    for (int j = 0; j < A_LOADS; ++j) a_src[j] += (size_t)kt_begin * BK;
+#pragma unroll
+    for (int j = 0; j < B_LOADS; ++j) b_src[j] += (size_t)kt_begin * BK;
+#pragma unroll
+    for (int s = 0; s < STAGES - 1; ++s)
+        if (s < KT) issue_loads(s, s);
+
+    // Wait until tile kt has landed in LDS for every wavefront.  Tiles requested after kt
+    // (at most STAGES-2 of them) may stay in flight.
+    auto sync_for = [&](int kt) {
+        const int ahead = (KT - 1 - kt) < (STAGES - 2) ? (KT - 1 - kt) : (STAGES - 2);
+        if constexpr (STAGES == 2) {
+            wait_vmcnt_and_barrier<0>();
+        } else if constexpr (STAGES == 3) {
+            if (ahead >= 1) wait_vmcnt_and_barrier<LPW>(); else wait_vmcnt_and_barrier<0>();
+        } else {
+            if (ahead >= 2) wait_vmcnt_and_barrier<2 * LPW>();
+            else if (ahead == 1) wait_vmcnt_and_barrier<LPW>();
+            else wait_vmcnt_and_barrier<0>();
+        }
+    };
+    auto load_frags = [&](half8_t (&af)[MT], half8_t (&bf)[NT], int kt, int ks) {
+        const unsigned char* st = smem_raw + (kt % STAGES) * STAGE_BYTES;
+#pragma unroll
+        for (int i = 0; i < MT; ++i)
+            af[i] = *reinterpret_cast<const half8_t*>(st + a_base + i * 32 * RB + fr_off[ks]);
+#pragma unroll
+        for (int j = 0; j < NT; ++j)
+            bf[j] = *reinterpret_cast<const half8_t*>(st + b_base + j * 32 * RB + fr_off[ks]);
+    };
+    auto mfmas = [&](const half8_t (&af)[MT], const half8_t (&bf)[NT]) {
+#if defined(TL_EXP_NOMFMA)
+        acc[0][0][0] += (float)af[0][0] + (float)bf[0][0];
+        return;
+#endif
+#pragma unroll
+        for (int i = 0; i < MT; ++i)
+#pragma unroll
+            for (int j = 0; j < NT; ++j)
+                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[i], bf[j], acc[i][j], 0, 0, 0);
+    };
+
+    if constexpr (PIPE) {
+        // Fragments are double buffered in registers: the ds_reads of K step s+1 (or of the
+        // next tile's first step, after the tile barrier) are issued before the MFMAs of step s.
+        static_assert(KS % 2 == 0, "fragment ping-pong needs an even number of K steps");
+        half8_t af[2][MT], bf[2][NT];
+        sync_for(0);
+        if (STAGES - 1 < KT) issue_loads((STAGES - 1) % STAGES, STAGES - 1);
+        load_frags(af[0], bf[0], 0, 0);
+        for (int kt = 0; kt < KT; ++kt) {
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) {
+                const int cur = ks & 1, nxt = cur ^ 1;
+                if (ks + 1 < KS) {
+                    load_frags(af[nxt], bf[nxt], kt, ks + 1);
+                } else if (kt + 1 < KT) {
+                    sync_for(kt + 1);  // every wavefront holds its last fragments of tile kt in registers
+                    if (kt + STAGES < KT) issue_loads((kt + STAGES) % STAGES, kt + STAGES);
+                    load_frags(af[nxt], bf[nxt], kt + 1, 0);
+                }
+                mfmas(af[cur], bf[cur]);
+            }
+        }
+    } else {
+        for (int kt = 0; kt < KT; ++kt) {
+            sync_for(kt);
+            if (kt + STAGES - 1 < KT) issue_loads((kt + STAGES - 1) % STAGES, kt + STAGES - 1);
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) {
+                half8_t af[MT], bf[NT];
+                load_frags(af, bf, kt, ks);
+                mfmas(af, bf);
+            }
+        }
+    }
+
+    const int c_col = lane & 31;
+    const int c_row_base = (lane >> 5) * 4;
+#pragma unroll
+    for (int i = 0; i < MT; ++i) {
+#pragma unroll
+        for (int j = 0; j < NT; ++j) {
+            const int col = n0 + wn * TN + j * 32 + c_col;
+            if (col >= N) continue;
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                const int row = m0 + wm * TM + i * 32 + 8 * (e / 4) + c_row_base + (e % 4);
+#if defined(TL_EXP_NOSTORE)
+                if (row < M && acc[i][j][e] == 123.456f) C[(size_t)row * N + col] = (half_t)acc[i][j][e];
+#else
+                if (row < M) {
+                    if (a.partial)
+                        a.partial[((size_t)blockIdx.z * M + row) * N + col] = acc[i][j][e];
+                    else
+                        C[(size_t)row * N + col] = (half_t)acc[i][j][e];
+                }
+#endif
+            }
+        }
+    }
+}
+
+// out[i] = half(sum over splits, in split order, of partial[s][i]): second pass of split-K.
+__global__ void __launch_bounds__(256)
+splitk_reduce_kernel(half_t* __restrict__ out, const float* __restrict__ partial, size_t n, int splits) {
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (size_t i = ((size_t)blockIdx.x * blockDim.x + threadIdx.x) * 4; i < n; i += stride * 4) {
+        if (i + 4 <= n) {
+            float4_t v = *reinterpret_cast<const float4_t*>(partial + i);
+            for (int s = 1; s < splits; ++s) v += *reinterpret_cast<const float4_t*>(partial + (size_t)s * n + i);
+            half4_t h = {(half_t)v[0], (half_t)v[1], (half_t)v[2], (half_t)v[3]};
+            *reinterpret_cast<half4_t*>(out + i) = h;
+        } else {
+            for (size_t j = i; j < n; ++j) {
+                float v = partial[j];
+                for (int s = 1; s < splits; ++s) v += partial[(size_t)s * n + j];
+                out[j] = (half_t)v;
+            }
+        }
+    }
+}
+
 // Any shape, any alignment: 16x16 outputs per 256-thread workgroup through LDS tiles,
 // fp32 accumulation.  Correctness path for K % 8 != 0 or unaligned operands.
 template <typename T, typename AccOut>
@@ -209,14 +454,21 @@ gemm_generic_kernel(const T* __restrict__ A0, const T* __restrict__ B0, T* __res
 struct HgemmVariant {
     const char* name;
     int bm, bn, bk, threads;
+    int stages;  // 0: register-staged kernel (any K % 8 == 0); >= 2: direct-to-LDS ring (K % bk == 0)
     void (*kernel)(HgemmArgs);
 };
 
 #define TL_HGEMM_VARIANT(BM, BN, BK, WM, WN) \
-    { "t" #BM "x" #BN "x" #BK "w" #WM "x" #WN, BM, BN, BK, WM * WN * 64, hgemm_f16_mfma_kernel<BM, BN, BK, WM, WN> }
+    { "t" #BM "x" #BN "x" #BK "w" #WM "x" #WN, BM, BN, BK, WM * WN * 64, 0, hgemm_f16_mfma_kernel<BM, BN, BK, WM, WN> }
+#define TL_HGEMM_DLDS(BM, BN, BK, WM, WN, ST) \
+    { "d" #BM "x" #BN "x" #BK "w" #WM "x" #WN "s" #ST, BM, BN, BK, WM * WN * 64, ST, \
+      hgemm_f16_dlds_kernel<BM, BN, BK, WM, WN, ST, false> }
+#define TL_HGEMM_PIPE(BM, BN, BK, WM, WN, ST) \
+    { "p" #BM "x" #BN "x" #BK "w" #WM "x" #WN "s" #ST, BM, BN, BK, WM * WN * 64, ST, \
+      hgemm_f16_dlds_kernel<BM, BN, BK, WM, WN, ST, true> }
 
 static const HgemmVariant g_variants[] = {
-    {"auto", 0, 0, 0, 0, nullptr},
+    {"auto", 0, 0, 0, 0, 0, nullptr},
     TL_HGEMM_VARIANT(128, 128, 64, 2, 2),  // 1
     TL_HGEMM_VARIANT(256, 128, 64, 2, 2),  // 2
     TL_HGEMM_VARIANT(128, 256, 64, 2, 2),  // 3
@@ -225,23 +477,92 @@ static const HgemmVariant g_variants[] = {
     TL_HGEMM_VARIANT(256, 256, 32, 2, 2),  // 6
     TL_HGEMM_VARIANT(128, 128, 32, 2, 2),  // 7
     TL_HGEMM_VARIANT(64, 128, 64, 2, 2),   // 8
+    TL_HGEMM_VARIANT(256, 256, 64, 2, 4),  // 9   8 wavefronts, 128x64 each
+    TL_HGEMM_VARIANT(256, 256, 64, 4, 2),  // 10  8 wavefronts, 64x128 each
+    TL_HGEMM_VARIANT(256, 256, 32, 2, 4),  // 11
+    TL_HGEMM_VARIANT(256, 128, 64, 2, 4),  // 12  128x32 each
+    TL_HGEMM_VARIANT(256, 128, 64, 4, 2),  // 13  64x64 each
+    TL_HGEMM_VARIANT(128, 256, 64, 2, 4),  // 14  64x64 each
+    TL_HGEMM_VARIANT(128, 128, 64, 2, 4),  // 15  64x32 each
+    TL_HGEMM_DLDS(256, 256, 64, 2, 4, 2),  // 16
+    TL_HGEMM_DLDS(256, 256, 64, 2, 2, 2),  // 17
+    TL_HGEMM_DLDS(256, 256, 32, 2, 4, 4),  // 18
+    TL_HGEMM_DLDS(256, 256, 32, 2, 4, 3),  // 19
+    TL_HGEMM_DLDS(256, 256, 32, 2, 2, 4),  // 20
+    TL_HGEMM_DLDS(256, 128, 64, 2, 4, 3),  // 21
+    TL_HGEMM_DLDS(256, 128, 64, 2, 2, 3),  // 22
+    TL_HGEMM_DLDS(128, 256, 64, 2, 4, 3),  // 23
+    TL_HGEMM_DLDS(128, 128, 64, 2, 2, 4),  // 24
+    TL_HGEMM_DLDS(128, 128, 64, 2, 2, 2),  // 25
+    TL_HGEMM_DLDS(256, 128, 32, 2, 4, 4),  // 26
+    TL_HGEMM_DLDS(128, 128, 32, 2, 2, 4),  // 27
+    TL_HGEMM_PIPE(256, 256, 64, 2, 4, 2),  // 28
+    TL_HGEMM_PIPE(256, 256, 64, 2, 2, 2),  // 29
+    TL_HGEMM_PIPE(256, 128, 64, 2, 4, 2),  // 30
+    TL_HGEMM_PIPE(128, 256, 64, 2, 4, 2),  // 31
+    TL_HGEMM_PIPE(128, 256, 64, 2, 4, 3),  // 32
+    TL_HGEMM_PIPE(128, 128, 64, 2, 2, 2),  // 33
+    TL_HGEMM_PIPE(256, 128, 64, 2, 2, 2),  // 34
+    TL_HGEMM_PIPE(128, 256, 64, 2, 2, 2),  // 35
+    TL_HGEMM_PIPE(128, 128, 64, 2, 4, 2),  // 36
+    TL_HGEMM_PIPE(256, 256, 32, 2, 4, 4),  // 37
 };
 static constexpr int kNumVariants = sizeof(g_variants) / sizeof(g_variants[0]);
 static int g_forced_variant = 0;
 static bool g_attr_set[kNumVariants] = {false};
 
+static int g_forced_splits = 0;  // 0 = automatic
+
+// Library-owned fp32 workspace for split-K partial sums, grown on demand (stream-ordered reuse).
+static std::mutex g_ws_mu;
+static float* g_ws = nullptr;
+static size_t g_ws_floats = 0;
+static int hgemm_workspace(size_t floats, float** out) {
+    std::lock_guard<std::mutex> lk(g_ws_mu);
+    if (floats > g_ws_floats) {
+        if (g_ws) {
+            TL_HIP_TRY(hipStreamSynchronize(stream()));
+            TL_HIP_TRY(hipFree(g_ws));
+            g_ws = nullptr;
+            g_ws_floats = 0;
+        }
+        const size_t want = floats < (size_t)(8u << 20) ? (size_t)(8u << 20) : floats;
+        hipError_t e = hipMalloc((void**)&g_ws, want * sizeof(float));
+        if (e != hipSuccess) {
+            (void)hipGetLastError();
+            return set_error(TL_ENOMEM, "split-K workspace: hipMalloc(%zu bytes) failed: %s", want * sizeof(float),
+                             hipGetErrorString(e));
+        }
+        g_ws_floats = want;
+    }
+    *out = g_ws;
+    return TL_OK;
+}
+
 static size_t lds_bytes(const HgemmVariant& v) {
+    if (v.stages > 0) return (size_t)v.stages * (v.bm + v.bn) * v.bk * sizeof(half_t);
     return (size_t)2 * (v.bm + v.bn) * (v.bk + kPad) * sizeof(half_t);
 }
 
+static int hgemm_variant_index(const char* name) {
+    for (int i = 0; i < kNumVariants; ++i)
+        if (strcmp(g_variants[i].name, name) == 0) return i;
+    return 1;
+}
+
+// Measured on MI355X over the Llama2-7B prefill shapes (M in {128,512,2048}):
+//   >= ~0.9 x CUs tiles of 256x256 : 256x256x64, 8 wavefronts (128x64 each), 2-stage LDS ring
+//   M >= 1024 otherwise            : 128x256x64, 8 wavefronts, fragments double buffered
+//   fewer rows                     : 128x128x64, 8 wavefronts, plus split-K (see launch_hgemm)
 static int pick_variant(size_t M, size_t N, size_t K, int cus) {
+    static const int v_big = hgemm_variant_index("d256x256x64w2x4s2");
+    static const int v_mid = hgemm_variant_index("p128x256x64w2x4s2");
+    static const int v_small = hgemm_variant_index("p128x128x64w2x4s2");
     (void)K;
     auto tiles = [&](int bm, int bn) { return ((M + bm - 1) / bm) * ((N + bn - 1) / bn); };
-    if (M <= 64) return 8;
-    if (tiles(256, 256) >= (size_t)cus * 2) return 4;
-    if (tiles(256, 128) >= (size_t)cus && M >= 256) return 2;
-    if (tiles(128, 128) >= (size_t)cus / 2) return 1;
-    return 5;
+    if (tiles(256, 256) * 10 >= (size_t)cus * 9) return v_big;
+    if (M >= 1024) return v_mid;
+    return v_small;
 }
 
 int launch_hgemm(const void* A, const void* B, void* C, size_t M, size_t N, size_t K, size_t batch, size_t sa,
@@ -267,7 +588,8 @@ int launch_hgemm(const void* A, const void* B, void* C, size_t M, size_t N, size
         TL_CHECK_LAUNCH("gemm_generic_kernel<half>");
         return TL_OK;
     }
-    const int vi = g_forced_variant ? g_forced_variant : pick_variant(M, N, K, device_info().cu_count);
+    int vi = g_forced_variant ? g_forced_variant : pick_variant(M, N, K, device_info().cu_count);
+    if (g_variants[vi].stages > 0 && K % g_variants[vi].bk != 0) vi = 1;  // direct-to-LDS path cannot zero-fill a K tail
     const HgemmVariant& v = g_variants[vi];
     const size_t lds = lds_bytes(v);
     if (lds > 64 * 1024 && !g_attr_set[vi]) {
@@ -289,8 +611,43 @@ int launch_hgemm(const void* A, const void* B, void* C, size_t M, size_t N, size
     a.sc = (long)sc;
     const size_t nblocks = (size_t)a.tiles_m * a.tiles_n;
     TL_REQUIRE(nblocks <= 0x7fffffffu, "hgemm: too many tiles");
-    hipLaunchKernelGGL(v.kernel, dim3((unsigned)nblocks, (unsigned)batch), dim3(v.threads), lds, st, a);
+    a.kt_per_split = 0x7fffffff;
+    a.partial = nullptr;
+    int splits = 1;
+    if (v.stages > 0) {
+        // Split K when the tile grid alone cannot occupy the chip (prefill with few tokens: the
+        // problem is then bound by streaming W, and every CU has to pull on it).
+        const int KT = (int)(K / v.bk);
+        const int cus = device_info().cu_count;
+        splits = g_forced_splits;
+        if (splits <= 0) {
+            // aim at ~1.5 workgroups per CU, keep at least 8 K tiles per split
+            splits = (int)(((size_t)cus * 3 / 2) / nblocks);
+            const int max_by_k = KT / 8 > 0 ? KT / 8 : 1;
+            if (splits > max_by_k) splits = max_by_k;
+            if (splits > 16) splits = 16;
+            if (splits < 1) splits = 1;
+        }
+        if (splits > KT) splits = KT;
+        if (batch != 1) splits = 1;
+        if (splits > 1) {
+            a.kt_per_split = (KT + splits - 1) / splits;
+            splits = (KT + a.kt_per_split - 1) / a.kt_per_split;
+            int rc = hgemm_workspace((size_t)splits * M * N, &a.partial);
+            if (rc != TL_OK) return rc;
+        }
+    }
+    hipLaunchKernelGGL(v.kernel, dim3((unsigned)nblocks, (unsigned)batch, (unsigned)splits), dim3(v.threads), lds, st, a);
     TL_CHECK_LAUNCH(v.name);
+    if (splits > 1) {
+        const size_t n = M * N;
+        size_t blocks = (n / 4 + 255) / 256;
+        const size_t cap = (size_t)device_info().cu_count * 8;
+        if (blocks > cap) blocks = cap;
+        if (blocks == 0) blocks = 1;
+        hipLaunchKernelGGL(splitk_reduce_kernel, dim3((unsigned)blocks), dim3(256), 0, st, (half_t*)C, a.partial, n, splits);
+        TL_CHECK_LAUNCH("splitk_reduce_kernel");
+    }
     return TL_OK;
 }
 
@@ -337,6 +694,12 @@ int tl_set_hgemm_variant(int variant) {
     TL_REQUIRE(variant >= 0 && variant < tl::kNumVariants, "tl_set_hgemm_variant: %d out of range [0,%d)",
                variant, tl::kNumVariants);
     tl::g_forced_variant = variant;
+    return TL_OK;
+}
+
+int tl_set_hgemm_splits(int splits) {
+    TL_REQUIRE(splits >= 0 && splits <= 64, "tl_set_hgemm_splits: %d out of range [0,64]", splits);
+    tl::g_forced_splits = splits;
     return TL_OK;
 }
 

@@ -138,7 +138,8 @@ def test_hgemm_prefill_shapes_sampled(dev, oracle, M, N, K):
 def test_hgemm_every_variant_ragged(dev, oracle):
     names = dev.hgemm_variants()
     for v in range(1, len(names)):
-        for (M, N, K) in [(300, 500, 264), (2, 3, 8), (129, 257, 72), (64, 64, 64), (257, 130, 1000)]:
+        for (M, N, K) in [(300, 500, 264), (2, 3, 8), (129, 257, 72), (64, 64, 64), (257, 130, 1000), (300, 517, 256),
+                          (1, 9, 64), (513, 255, 128), (260, 1030, 192)]:
             _hgemm_case(dev, oracle, M, N, K, seed=1000 + v, variant=v, b_std=0.1)
 
 
