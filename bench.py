@@ -11,8 +11,12 @@ Prints ONE JSON line.  `value` = algorithmic bytes of a step / wall time of a st
 decimal).  `roofline` = the GEMV kernel against the 8 TB/s HBM peak, from a HIP event pair
 recorded on the launch stream around the timed region.  `cpu_baseline` = the CPU oracle
 (a port of the reference's OpenMP CPU<half>::matmul2d) timed on this host on the same sweep.
-`extra` carries per-shape GEMV numbers, prefill HGEMM TFLOP/s and, when the C++ driver is
-built, Llama2-7B decode tok/s.
+`extra` carries per-shape GEMV numbers, prefill HGEMM TFLOP/s (against the published MFMA peak and
+against the MFMA rate this chip sustains out of registers) and Llama2-7B decode tok/s.
+
+`--workload hgemm` times only the prefill HGEMM shapes (step = one pass over the M=2048 shapes)
+and prints the same kind of line with an MFMA roofline; it exists so that the MFMA profile under
+profiles/ can be taken from a committed command.
 """
 from __future__ import annotations
 
@@ -30,7 +34,7 @@ HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
 MFMA_FP16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16 MFMA, published
 
 SWEEP = [(4096, 4096), (11008, 4096), (4096, 11008), (32000, 4096)]
-# prefill shapes reported in `extra` (M, N, K)
+# prefill shapes (M, N, K)
 HGEMM_SHAPES = [(2048, 4096, 4096), (2048, 11008, 4096), (2048, 32000, 4096), (2048, 4096, 11008),
                 (512, 4096, 4096), (512, 11008, 4096), (512, 32000, 4096), (512, 4096, 11008),
                 (128, 4096, 4096), (128, 11008, 4096), (128, 32000, 4096), (128, 4096, 11008)]
@@ -46,6 +50,7 @@ def parse_args():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--workload", choices=["gemv", "hgemm"], default="gemv")
     ap.add_argument("--no-extra", action="store_true", help="skip the HGEMM / per-shape / model extras")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--copy-calibration", action="store_true",
@@ -54,7 +59,7 @@ def parse_args():
     return ap.parse_args()
 
 
-def cpu_baseline(budget_s: float = 10.0):
+def cpu_baseline_gemv(budget_s: float = 10.0):
     """Time the CPU oracle on the full decode sweep (all four shapes, every row)."""
     import numpy as np
     from oracle import oracle
@@ -82,6 +87,31 @@ def cpu_baseline(budget_s: float = 10.0):
     }
 
 
+def cpu_baseline_hgemm():
+    """Time the CPU oracle on 16 rows of X of the 2048x4096x4096 prefill GEMM (0.27 G multiply-adds)."""
+    import numpy as np
+    from oracle import oracle
+    from tensorlib_amd import synth
+    rows, N, K = 16, 4096, 4096
+    A = synth.normal_f16(30, (rows, K), 1.0)
+    B = synth.normal_f16(31, (N, K), 0.02)
+    oracle.matmul2d(A, B)
+    times = []
+    for _ in range(7):
+        t0 = time.perf_counter()
+        oracle.matmul2d(A, B)
+        times.append(time.perf_counter() - t0)
+    med = float(np.median(times))
+    return {
+        "value": round(2.0 * rows * N * K / med / 1e12, 5),
+        "unit": "TFLOP/s",
+        "cores": oracle.max_threads(),
+        "kind": "port",
+        "sample": f"{rows} rows of X of the 2048x4096x4096 shape ({rows}x{N}x{K}), median of 7 runs, "
+                  f"{med * 1e3:.1f} ms; full shape would take {med * 2048 / rows:.2f} s (extrapolated)",
+    }
+
+
 def time_region(fn, reps: int, torch):
     """Run fn() reps times between a HIP event pair on the current (= library) stream; returns
     (wall seconds, event seconds)."""
@@ -96,6 +126,40 @@ def time_region(fn, reps: int, torch):
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
     return wall, e0.elapsed_time(e1) * 1e-3
+
+
+def mfma_sustained(dev):
+    """MFMA rate out of registers: constant operands vs operands changing with every instruction."""
+    import ctypes
+    out = {}
+    for name, mode in (("constant_operands", 0), ("changing_operands", 1)):
+        v = ctypes.c_double()
+        from tensorlib_amd._lib import check
+        check(dev.lib.tl_measure_mfma_rate_f16(mode, ctypes.byref(v)), "tl_measure_mfma_rate_f16")
+        out[name] = round(v.value, 1)
+    return out
+
+
+def hgemm_table(dev, randn, torch, synth, sustained_tf):
+    hg = {}
+    for (M, N, K) in HGEMM_SHAPES:
+        A = randn((M, K), 1.0)
+        B = randn((N, K), 0.02)
+        C = torch.empty((M, N), device="cuda", dtype=torch.float16)
+        for _ in range(3):
+            dev.matmul2d(A, B, C)
+        reps = 20
+        _, ev1 = time_region(lambda: dev.matmul2d(A, B, C), reps, torch)
+        us = ev1 / reps * 1e6
+        tf = synth.gemm_flops(M, N, K) / us / 1e6
+        ai = synth.gemm_flops(M, N, K) / synth.gemm_min_bytes(M, N, K)
+        bound_tf = min(MFMA_FP16_PEAK_TFLOPS, ai * HBM_PEAK_GBS / 1e3)
+        hg[f"{M}x{N}x{K}"] = {"us": round(us, 1), "TFLOP/s": round(tf, 1),
+                              "frac_mfma_peak": round(tf / MFMA_FP16_PEAK_TFLOPS, 4),
+                              "bound": "mfma" if bound_tf >= MFMA_FP16_PEAK_TFLOPS else "hbm",
+                              "frac_of_bound": round(tf / bound_tf, 4),
+                              "frac_of_sustained_mfma": round(tf / sustained_tf, 4)}
+    return hg
 
 
 def main():
@@ -117,6 +181,41 @@ def main():
 
     def randn(shape, std):
         return (torch.randn(shape, generator=gen, device="cuda", dtype=torch.float32) * std).to(torch.float16)
+
+    if args.workload == "hgemm":
+        shapes = [s for s in HGEMM_SHAPES if s[0] == 2048]
+        mats = [(randn((M, K), 1.0), randn((N, K), 0.02), torch.empty((M, N), device="cuda", dtype=torch.float16))
+                for (M, N, K) in shapes]
+        step_flops = sum(synth.gemm_flops(*s) for s in shapes)
+
+        def step():
+            for A, B, C in mats:
+                dev.matmul2d(A, B, C)
+        for _ in range(args.warmup):
+            step()
+        wall, ev = time_region(step, args.steps, torch)
+        value = step_flops / (wall / args.steps) / 1e12
+        achieved = step_flops / (ev / args.steps) / 1e12
+        sustained = mfma_sustained(dev)
+        out = {
+            "metric": "fp16 HGEMM TFLOP/s (Llama2-7B prefill, M=2048 shapes)",
+            "value": round(value, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+            "ms_per_step": round(wall * 1e3 / args.steps, 5), "higher_is_better": True, "scaling": "weak",
+            "vs_baseline": None, "dtype": "f16", "data": "synthetic",
+            "config": {"workload": "prefill HGEMM X[2048,K] . W[N,K]^T for (N,K) in 4096x4096, 11008x4096, 32000x4096, "
+                                   "4096x11008; X~N(0,1), W~N(0,0.02); fp32 accumulate", "flops_per_step": step_flops},
+            "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": MFMA_FP16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                         "frac": round(achieved / MFMA_FP16_PEAK_TFLOPS, 4), "traffic": None,
+                         "kernel": "hgemm_f16_dlds_kernel", "flops_per_launch": step_flops / len(shapes),
+                         "avg_launch_us": round(ev / args.steps / len(shapes) * 1e6, 2),
+                         "sustained_mfma_tflops": sustained},
+        }
+        if not args.no_extra:
+            out["extra"] = {"hgemm_prefill": hgemm_table(dev, randn, torch, synth, sustained["changing_operands"])}
+        if not args.no_cpu:
+            out["cpu_baseline"] = cpu_baseline_hgemm()
+        print(json.dumps(out))
+        return
 
     # ---- weights: NSETS rotating sets of the four matrices (3 x 476 MB) ------------------
     NSETS = 3
@@ -179,6 +278,8 @@ def main():
             "avg_launch_us": round(avg_launch_s * 1e6, 3),
         },
     }
+    del sets
+    torch.cuda.empty_cache()
 
     extra = {}
     if not args.no_extra:
@@ -204,33 +305,16 @@ def main():
         extra["gemv_per_shape"] = per_shape
         torch.cuda.empty_cache()
 
-        hg = {}
-        for (M, N, K) in HGEMM_SHAPES:
-            A = randn((M, K), 1.0)
-            B = randn((N, K), 0.02)
-            C = torch.empty((M, N), device="cuda", dtype=torch.float16)
-            for _ in range(3):
-                dev.matmul2d(A, B, C)
-            reps = 20
-            _, ev1 = time_region(lambda: dev.matmul2d(A, B, C), reps, torch)
-            us = ev1 / reps * 1e6
-            tf = synth.gemm_flops(M, N, K) / us / 1e6
-            ai = synth.gemm_flops(M, N, K) / synth.gemm_min_bytes(M, N, K)
-            bound_tf = min(MFMA_FP16_PEAK_TFLOPS, ai * HBM_PEAK_GBS / 1e3)
-            hg[f"{M}x{N}x{K}"] = {"us": round(us, 1), "TFLOP/s": round(tf, 1),
-                                  "frac_mfma_peak": round(tf / MFMA_FP16_PEAK_TFLOPS, 4),
-                                  "bound": "mfma" if bound_tf >= MFMA_FP16_PEAK_TFLOPS else "hbm",
-                                  "frac_of_bound": round(tf / bound_tf, 4)}
-        extra["hgemm_prefill"] = hg
-        try:
-            from tensorlib_amd import llama2
-            extra["llama2_7b_decode"] = llama2.bench_decode(dev)
-        except ImportError:
-            pass
+        sustained = mfma_sustained(dev)
+        extra["mfma_sustained_tflops"] = sustained
+        extra["hgemm_prefill"] = hgemm_table(dev, randn, torch, synth, sustained["changing_operands"])
+        torch.cuda.empty_cache()
+        from tensorlib_amd import llama2
+        extra["llama2_7b_decode"] = llama2.bench_decode(dev)
     out["extra"] = extra
 
     if not args.no_cpu:
-        out["cpu_baseline"] = cpu_baseline()
+        out["cpu_baseline"] = cpu_baseline_gemv()
     print(json.dumps(out))
 
 

@@ -106,6 +106,10 @@ int tl_set_gemv_variant(int variant);
 int tl_set_hgemm_variant(int variant);
 const char* tl_gemv_variant_name(int variant);
 const char* tl_hgemm_variant_name(int variant);
+/* Measurement hook (no reference counterpart): fp16 MFMA rate sustained out of registers, in
+ * TFLOP/s.  mode 0: constant operands; mode 1: both operands change with every instruction.
+ * Synchronises the stream.  Used by bench.py to place HGEMM against the power-managed ceiling. */
+int tl_measure_mfma_rate_f16(int mode, double* tflops);
 /* Tuning hook: force the number of K splits of the MFMA GEMM (0 = automatic). */
 int tl_set_hgemm_splits(int splits);
 /* Tuning hook: cap the GEMV grid at `waves` resident wavefronts per compute unit (0 = default). */
