@@ -66,6 +66,14 @@ int tlm_destroy(tlm_model* m);
 
 int tlm_set_weight(tlm_model* m, int kind, int layer, const void* dev_ptr);
 
+/* Create a model from a llama2.c legacy fp16 checkpoint, the file the reference's read_checkpoint
+ * loads (model/llama2_7b/src/main.cpp:36-228; writer script/export.py:138-190).  The model owns
+ * the weight memory.  max_seq_len > 0 caps the KV cache below the file's seq_len. */
+int tlm_load_checkpoint(const char* path, int max_tokens, int max_seq_len, tlm_model** out);
+
+/* out7 = {dim, hidden_dim, n_layers, n_heads, vocab_size, max_seq_len, max_tokens}. */
+int tlm_get_config(tlm_model* m, int* out7);
+
 /* Forward `n_tokens` tokens (device int32 ids) at positions [start_pos, start_pos + n_tokens).
  * all_logits != 0: logits for every token ([n_tokens, vocab], as Transformer::forward does);
  * all_logits == 0: only the last token's row is projected.  *logits_out receives the device

@@ -75,6 +75,7 @@ struct tlm_model {
     std::vector<LayerWeights> layers;
     std::vector<Buf> cache_k, cache_v;  // per layer [max_seq, n_heads, head_dim]
     Buf x, x_norm, x_residual, qkv, x13, x2, scores, scores2, mask, xq_c, keys_c, values_c, s_v, o_c, logits;
+    std::vector<void*> owned_weights;  // device allocations made by tlm_load_checkpoint
     int* d_tokens = nullptr;   // [max_tokens + generated]
     int d_tokens_cap = 0;
     Dev scratch_dev;           // method holder for calls that take explicit pointers
@@ -202,7 +203,9 @@ struct tlm_model {
         if (start_pos < 0 || start_pos + S > max_seq) throw std::runtime_error("positions exceed max_seq_len");
         // tok_embeddings.forward                                             Transformer.cpp:274
         ck(tl_embedding_f16(x.p, tok_emb, dev_tokens, S, dim, vocab), "embedding");
-        if (mode == TLM_MODE_FUSED && S == 1) {
+        // the fused attention kernel covers head_dim 64/128/256; other sizes take the reference chain
+        const bool fused_ok = head_dim == 64 || head_dim == 128 || head_dim == 256;
+        if (mode == TLM_MODE_FUSED && S == 1 && fused_ok) {
             decode_fused(start_pos);   // leaves rmsnorm(x) * final_norm in x_norm
             gemv(x_norm.p, classifier, logits.p, vocab, dim);
             return logits.p;
@@ -277,7 +280,108 @@ int tlm_destroy(tlm_model* m) {
                    &m->xq_c, &m->keys_c, &m->values_c, &m->s_v, &m->o_c, &m->logits})
         b->release();
     if (m->d_tokens) tl_free(m->d_tokens);
+    for (void* p : m->owned_weights) tl_free(p);
     delete m;
+    return 0;
+}
+
+// Reader of the llama2.c "legacy" fp16 checkpoint the reference loads
+// (model/llama2_7b/src/main.cpp:26-34 header, :36-190 tensor order, written by
+// script/export.py:138-190): 7 int32 (dim, hidden_dim, n_layers, n_heads, n_kv_heads,
+// +-vocab_size, seq_len; vocab_size > 0 means the classifier shares the embedding), then fp16
+// tensors: tok_emb, att_norm[L], wq[L], wk[L], wv[L], wo[L], ffn_norm[L], w1[L], w2[L], w3[L],
+// final norm, seq_len*head_dim halves of rotary tables (skipped, as the reference skips them),
+// classifier unless shared.  Each layer's wq|wk|wv and w1|w3 are placed adjacently in HBM so the
+// fused decode mode can run them as single GEMVs.
+int tlm_load_checkpoint(const char* path, int max_tokens, int max_seq_len, tlm_model** out) {
+    if (!path || !out) return fail("tlm_load_checkpoint: null argument");
+    *out = nullptr;
+    FILE* f = fopen(path, "rb");
+    if (!f) return fail("tlm_load_checkpoint: cannot open %s", path);
+    int hdr[7];
+    if (fread(hdr, sizeof(int), 7, f) != 7) { fclose(f); return fail("tlm_load_checkpoint: short header in %s", path); }
+    const int dim = hdr[0], hidden = hdr[1], L = hdr[2], heads = hdr[3], kv_heads = hdr[4];
+    const bool shared = hdr[5] > 0;
+    const int vocab = hdr[5] < 0 ? -hdr[5] : hdr[5];
+    const int seq_len = hdr[6];
+    if (dim <= 0 || hidden <= 0 || L <= 0 || heads <= 0 || vocab <= 0 || seq_len <= 0 || dim % heads != 0) {
+        fclose(f);
+        return fail("tlm_load_checkpoint: implausible header in %s", path);
+    }
+    if (kv_heads != heads) { fclose(f); return fail("tlm_load_checkpoint: n_kv_heads %d != n_heads %d (grouped-query attention is not in the reference model)", kv_heads, heads); }
+    const int use_seq = (max_seq_len > 0 && max_seq_len < seq_len) ? max_seq_len : seq_len;
+    tlm_model* m = nullptr;
+    int rc = tlm_create(&m, dim, hidden, L, heads, vocab, use_seq, 1e-5f, max_tokens < use_seq ? max_tokens : use_seq);
+    if (rc != 0) { fclose(f); return rc; }
+    std::vector<unsigned char> stage;
+    bool ok = true;
+    std::string err;
+    auto dev_alloc = [&](size_t elems) -> half* {
+        void* p = nullptr;
+        if (tl_malloc(&p, elems * sizeof(half)) != TL_OK) { ok = false; err = tl_last_error(); return nullptr; }
+        m->owned_weights.push_back(p);
+        return static_cast<half*>(p);
+    };
+    auto read_into = [&](half* dst, size_t elems) {
+        if (!ok) return;
+        stage.resize(elems * sizeof(half));
+        if (fread(stage.data(), sizeof(half), elems, f) != elems) { ok = false; err = "file too short"; return; }
+        if (tl_memcpy_h2d(dst, stage.data(), elems * sizeof(half)) != TL_OK) { ok = false; err = tl_last_error(); }
+    };
+    const size_t dd = (size_t)dim * dim, hd = (size_t)hidden * dim;
+    half* emb = dev_alloc((size_t)vocab * dim);
+    std::vector<half*> qkv(L), w13(L), wo(L), w2(L), an(L), fn(L);
+    for (int l = 0; l < L && ok; ++l) {
+        qkv[l] = dev_alloc(3 * dd); w13[l] = dev_alloc(2 * hd); wo[l] = dev_alloc(dd); w2[l] = dev_alloc(hd);
+        an[l] = dev_alloc(dim); fn[l] = dev_alloc(dim);
+    }
+    half* fnorm = dev_alloc(dim);
+    if (ok) {
+        read_into(emb, (size_t)vocab * dim);
+        for (int l = 0; l < L; ++l) read_into(an[l], dim);
+        for (int l = 0; l < L; ++l) read_into(qkv[l], dd);
+        for (int l = 0; l < L; ++l) read_into(qkv[l] + dd, dd);
+        for (int l = 0; l < L; ++l) read_into(qkv[l] + 2 * dd, dd);
+        for (int l = 0; l < L; ++l) read_into(wo[l], dd);
+        for (int l = 0; l < L; ++l) read_into(fn[l], dim);
+        for (int l = 0; l < L; ++l) read_into(w13[l], hd);
+        for (int l = 0; l < L; ++l) read_into(w2[l], hd);
+        for (int l = 0; l < L; ++l) read_into(w13[l] + hd, hd);
+        read_into(fnorm, dim);
+    }
+    half* cls = emb;
+    if (ok && !shared) {
+        if (fseek(f, (long)((size_t)seq_len * (dim / heads) * sizeof(half)), SEEK_CUR) != 0) { ok = false; err = "seek failed"; }
+        cls = dev_alloc((size_t)vocab * dim);
+        read_into(cls, (size_t)vocab * dim);
+    }
+    fclose(f);
+    if (!ok) {
+        tlm_destroy(m);
+        return fail("tlm_load_checkpoint: %s: %s", path, err.c_str());
+    }
+    tlm_set_weight(m, TLM_W_TOK_EMB, 0, emb);
+    tlm_set_weight(m, TLM_W_FINAL_NORM, 0, fnorm);
+    tlm_set_weight(m, TLM_W_CLASSIFIER, 0, cls);
+    for (int l = 0; l < L; ++l) {
+        tlm_set_weight(m, TLM_W_ATT_NORM, l, an[l]);
+        tlm_set_weight(m, TLM_W_WQ, l, qkv[l]);
+        tlm_set_weight(m, TLM_W_WK, l, qkv[l] + dd);
+        tlm_set_weight(m, TLM_W_WV, l, qkv[l] + 2 * dd);
+        tlm_set_weight(m, TLM_W_WO, l, wo[l]);
+        tlm_set_weight(m, TLM_W_FFN_NORM, l, fn[l]);
+        tlm_set_weight(m, TLM_W_W1, l, w13[l]);
+        tlm_set_weight(m, TLM_W_W2, l, w2[l]);
+        tlm_set_weight(m, TLM_W_W3, l, w13[l] + hd);
+    }
+    *out = m;
+    return 0;
+}
+
+int tlm_get_config(tlm_model* m, int* out7) {
+    if (!m || !out7) return fail("tlm_get_config: null argument");
+    out7[0] = m->dim; out7[1] = m->hidden; out7[2] = m->n_layers; out7[3] = m->n_heads;
+    out7[4] = m->vocab; out7[5] = m->max_seq; out7[6] = m->max_tokens;
     return 0;
 }
 

@@ -26,6 +26,8 @@ _PROTOS = {
     "tlm_forward": (_i, [_vp, _vp, _i, _i, _i, _i, ctypes.POINTER(_vp)]),
     "tlm_generate": (_i, [_vp, _vp, _i, _i, _i, _vp, ctypes.POINTER(ctypes.c_double), ctypes.POINTER(ctypes.c_double)]),
     "tlm_get_buffer": (_i, [_vp, _i, _i, ctypes.POINTER(_vp)]),
+    "tlm_load_checkpoint": (_i, [ctypes.c_char_p, _i, _i, ctypes.POINTER(_vp)]),
+    "tlm_get_config": (_i, [_vp, ctypes.POINTER(_i)]),
 }
 _llib = None
 
@@ -69,15 +71,56 @@ class Llama2Config:
         return 2 * (self.n_layers * per_layer + self.vocab_size * self.dim)
 
 
+def write_checkpoint(path: str, cfg: Llama2Config, w: dict, shared_classifier: bool = False) -> None:
+    """Write weights (name scheme of Llama2Model.set_weights) as a llama2.c legacy fp16 checkpoint:
+    the layout script/export.py:138-190 produces and model/llama2_7b/src/main.cpp:36-228 reads.
+    The rotary tables the format carries (seq_len * head_dim halves) are written as cos/sin of
+    pos * 10000^(-2i/head_dim); readers of this format skip them."""
+    import struct
+    L = cfg.n_layers
+    with open(path, "wb") as f:
+        vocab = cfg.vocab_size if shared_classifier else -cfg.vocab_size
+        f.write(struct.pack("iiiiiii", cfg.dim, cfg.hidden_dim, L, cfg.n_heads, cfg.n_heads, vocab, cfg.max_seq_len))
+
+        def put(a):
+            f.write(np.ascontiguousarray(a, dtype=np.float16).tobytes())
+        put(w["tok_emb"])
+        for name in ("att_norm", "wq", "wk", "wv", "wo", "ffn_norm", "w1", "w2", "w3"):
+            for l in range(L):
+                put(w[f"{name}.{l}"])
+        put(w["final_norm"])
+        half_d = cfg.head_dim // 2
+        ang = np.outer(np.arange(cfg.max_seq_len), 10000.0 ** (-np.arange(half_d) * 2.0 / cfg.head_dim))
+        put(np.cos(ang))
+        put(np.sin(ang))
+        if not shared_classifier:
+            put(w["classifier"])
+
+
 class Llama2Model:
-    def __init__(self, dev, cfg: Llama2Config, max_tokens: int):
+    def __init__(self, dev, cfg: Llama2Config, max_tokens: int, _handle=None):
         self.dev, self.cfg, self.max_tokens = dev, cfg, max_tokens
         self.l = llama2_lib()
+        self.weights = {}   # keeps the torch tensors alive
+        if _handle is not None:
+            self.h = _handle
+            return
         h = _vp()
         _ck(self.l.tlm_create(ctypes.byref(h), cfg.dim, cfg.hidden_dim, cfg.n_layers, cfg.n_heads, cfg.vocab_size,
                               cfg.max_seq_len, cfg.norm_eps, max_tokens), "tlm_create")
         self.h = h
-        self.weights = {}   # keeps the torch tensors alive
+
+    @classmethod
+    def from_checkpoint(cls, dev, path: str, max_tokens: int, max_seq_len: int = 0) -> "Llama2Model":
+        """Load a llama2.c legacy fp16 .bin (the file the reference's read_checkpoint loads)."""
+        l = llama2_lib()
+        h = _vp()
+        _ck(l.tlm_load_checkpoint(path.encode(), max_tokens, max_seq_len, ctypes.byref(h)), "tlm_load_checkpoint")
+        c7 = (ctypes.c_int * 7)()
+        _ck(l.tlm_get_config(h, c7), "tlm_get_config")
+        cfg = Llama2Config(dim=c7[0], hidden_dim=c7[1], n_layers=c7[2], n_heads=c7[3], vocab_size=c7[4],
+                           max_seq_len=c7[5])
+        return cls(dev, cfg, c7[6], _handle=h)
 
     def close(self):
         if self.h:

@@ -169,3 +169,49 @@ def test_llama2_7b_full_model(dev):
     assert np.array_equal(out_f, out_f2)
     print(f"7B decode: fused {255 / td_f:.1f} tok/s, chain {255 / td_c:.1f} tok/s; prefill {128 / tp_f:.0f} tok/s")
     m.close()
+
+
+def test_checkpoint_loader_round_trip(dev, tmp_path):
+    """A llama2.c legacy fp16 .bin written with the reference's tensor order must load into a model
+    whose logits are bit-identical to one built from the same arrays (both modes), for the
+    separate-classifier and the shared-classifier variants of the format."""
+    from tensorlib_amd.llama2 import MODE_FUSED, MODE_REFERENCE_CHAIN, Llama2Config, Llama2Model, write_checkpoint
+    cfg = Llama2Config(dim=128, hidden_dim=352, n_layers=2, n_heads=2, vocab_size=300, max_seq_len=32)
+    w = _weights(cfg, 5000)
+    toks = synth.token_ids(12, 6, cfg.vocab_size)
+    for shared in (False, True):
+        ws = dict(w)
+        if shared:
+            ws["classifier"] = ws["tok_emb"]
+        path = str(tmp_path / f"toy_{int(shared)}.bin")
+        write_checkpoint(path, cfg, ws, shared_classifier=shared)
+        m_file = Llama2Model.from_checkpoint(dev, path, max_tokens=8)
+        assert (m_file.cfg.dim, m_file.cfg.hidden_dim, m_file.cfg.n_layers, m_file.cfg.n_heads, m_file.cfg.vocab_size,
+                m_file.cfg.max_seq_len) == (128, 352, 2, 2, 300, 32)
+        m_mem = Llama2Model(dev, cfg, max_tokens=8)
+        m_mem.set_weights(ws)
+        for mode in (MODE_REFERENCE_CHAIN, MODE_FUSED):
+            a = m_file.forward(toks[:5], 0, mode).cpu().numpy()
+            b = m_mem.forward(toks[:5], 0, mode).cpu().numpy()
+            assert np.array_equal(a.view(np.uint16), b.view(np.uint16))
+            a = m_file.forward(toks[5:6], 5, mode).cpu().numpy()
+            b = m_mem.forward(toks[5:6], 5, mode).cpu().numpy()
+            assert np.array_equal(a.view(np.uint16), b.view(np.uint16))
+        m_file.close(), m_mem.close()
+
+
+def test_checkpoint_loader_rejects_bad_files(dev, tmp_path):
+    from tensorlib_amd import TensorLibError
+    from tensorlib_amd.llama2 import Llama2Config, Llama2Model, write_checkpoint
+    with pytest.raises(TensorLibError):
+        Llama2Model.from_checkpoint(dev, str(tmp_path / "missing.bin"), 4)
+    cfg = Llama2Config(dim=64, hidden_dim=128, n_layers=1, n_heads=2, vocab_size=50, max_seq_len=16)
+    path = str(tmp_path / "short.bin")
+    write_checkpoint(path, cfg, _weights(cfg, 6000))
+    data = open(path, "rb").read()
+    open(path, "wb").write(data[:len(data) // 2])       # truncated tensor section
+    with pytest.raises(TensorLibError):
+        Llama2Model.from_checkpoint(dev, path, 4)
+    open(path, "wb").write(data[:10])                    # truncated header
+    with pytest.raises(TensorLibError):
+        Llama2Model.from_checkpoint(dev, path, 4)
