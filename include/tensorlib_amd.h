@@ -181,6 +181,17 @@ int tl_silu_mul_f16(void* out, const void* a, const void* b, size_t n);
 int tl_decode_attention_f16(void* out, const void* q, const void* cache_k, const void* cache_v,
                             int T, int n_heads, int head_dim);
 
+/* y[N] = W[N,K] . (silu(ab[0:K]) * ab[K:2K]): FeedForward's silu, EwiseMul and w2 projection
+ * (model/llama2_7b/src/Transformer.cpp:137-143) in one launch; the gated vector is rounded to
+ * fp16 once, as tl_silu_mul_f16 would store it.  Needs 512 <= K <= 12288, K % 8 == 0. */
+int tl_gemv_silu_mul_f16(const void* ab, const void* W, void* y, size_t N, size_t K);
+
+/* tl_rope_qk_store_kv_f16 + tl_decode_attention_f16 in one launch pair: qkv is the raw q|k|v
+ * projection of the token at position `pos`; q is rotated on load, the rotated k and the v row
+ * are written to cache_k[pos] / cache_v[pos], and out[h,:] attends to positions 0..pos. */
+int tl_decode_attention_rope_f16(void* out, const void* qkv, void* cache_k, void* cache_v, int pos,
+                                 int n_heads, int head_dim);
+
 /* Decode-step glue after a fused q|k|v projection (qkv = [q | k | v], each n_heads*head_dim
  * halves): rotary-embed q in place, rotary-embed k into cache_k[pos], copy v into cache_v[pos]
  * (caches are [max_seq, n_heads, head_dim]).  Replaces two apply_rotary_emb launches and two

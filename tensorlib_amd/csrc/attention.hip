@@ -37,10 +37,30 @@ constexpr int kAttnThreads = 256;
 constexpr int kAttnChunk = 64;  // cached positions per workgroup
 
 // partial layout per (head, chunk): [0] = max, [1] = sum, [2 .. 2+head_dim) = sum_t p_t * V[t]
-template <int LPR>
+// Rotate the 4 (even, odd) pairs of one 16-byte chunk of a head vector; `d0` is the index of the
+// chunk's first element inside the head.  Same arithmetic as rope_kernel: fp32 angle, cos/sin
+// rounded to half, fp32 products, one rounding per output.
+__device__ __forceinline__ half8_t rope_chunk(half8_t v, int pos, int d0, int head_dim) {
+    half8_t r;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const float theta = (float)pos * 1.0f / powf(10000.0f, (float)(d0 + 2 * i) / (float)head_dim);
+        const float c = (float)(half_t)cosf(theta);
+        const float s = (float)(half_t)sinf(theta);
+        const float v0 = (float)v[2 * i], v1 = (float)v[2 * i + 1];
+        r[2 * i] = (half_t)(v0 * c - v1 * s);
+        r[2 * i + 1] = (half_t)(v0 * s + v1 * c);
+    }
+    return r;
+}
+
+// FUSE_ROPE: `q` points at the raw q|k|v projection of the new token (position T-1).  q is rotated
+// on load; the workgroup that owns the last chunk rotates the new k row, uses it, and writes it and
+// the new v row into the caches (each head's workgroup writes only its own head slice).
+template <int LPR, bool FUSE_ROPE>
 __global__ void __launch_bounds__(kAttnThreads)
-decode_attn_partial_kernel(half_t* out, float* partial, const half_t* q, const half_t* cache_k,
-                           const half_t* cache_v, int T, int n_heads, float inv_scale, int n_chunks) {
+decode_attn_partial_kernel(half_t* out, float* partial, const half_t* q, half_t* cache_k,
+                           half_t* cache_v, int T, int n_heads, float inv_scale, int n_chunks) {
     constexpr int D = LPR * 8;
     constexpr int GROUPS = kAttnThreads / LPR;
     __shared__ float sc[kAttnChunk];
@@ -56,11 +76,19 @@ decode_attn_partial_kernel(half_t* out, float* partial, const half_t* q, const h
     const int grp = tid / LPR;
     const size_t row_stride = (size_t)n_heads * D;
 
-    const half8_t qv = *reinterpret_cast<const half8_t*>(q + (size_t)h * D + sub * 8);
+    half8_t qv = *reinterpret_cast<const half8_t*>(q + (size_t)h * D + sub * 8);
+    if constexpr (FUSE_ROPE) qv = rope_chunk(qv, T - 1, sub * 8, D);
 
     // scores
     for (int t = t0 + grp; t < t1; t += GROUPS) {
-        const half8_t kv = *reinterpret_cast<const half8_t*>(cache_k + (size_t)t * row_stride + (size_t)h * D + sub * 8);
+        half8_t kv;
+        if (FUSE_ROPE && t == T - 1) {
+            kv = *reinterpret_cast<const half8_t*>(q + row_stride + (size_t)h * D + sub * 8);
+            kv = rope_chunk(kv, T - 1, sub * 8, D);
+            *reinterpret_cast<half8_t*>(cache_k + (size_t)t * row_stride + (size_t)h * D + sub * 8) = kv;
+        } else {
+            kv = *reinterpret_cast<const half8_t*>(cache_k + (size_t)t * row_stride + (size_t)h * D + sub * 8);
+        }
         float s = 0.f;
 #pragma unroll
         for (int i = 0; i < 8; ++i) s = __builtin_fmaf((float)qv[i], (float)kv[i], s);
@@ -103,7 +131,13 @@ decode_attn_partial_kernel(half_t* out, float* partial, const half_t* q, const h
 #pragma unroll
     for (int i = 0; i < 8; ++i) acc[i] = 0.f;
     for (int t = t0 + grp; t < t1; t += GROUPS) {
-        const half8_t vv = *reinterpret_cast<const half8_t*>(cache_v + (size_t)t * row_stride + (size_t)h * D + sub * 8);
+        half8_t vv;
+        if (FUSE_ROPE && t == T - 1) {
+            vv = *reinterpret_cast<const half8_t*>(q + 2 * row_stride + (size_t)h * D + sub * 8);
+            *reinterpret_cast<half8_t*>(cache_v + (size_t)t * row_stride + (size_t)h * D + sub * 8) = vv;
+        } else {
+            vv = *reinterpret_cast<const half8_t*>(cache_v + (size_t)t * row_stride + (size_t)h * D + sub * 8);
+        }
         const float p = sc[t - t0];
 #pragma unroll
         for (int i = 0; i < 8; ++i) acc[i] = __builtin_fmaf(p, (float)vv[i], acc[i]);
@@ -211,6 +245,59 @@ add_rms_norm_kernel(half_t* sum_out, half_t* norm_out, const half_t* a, const ha
         norm_out[base + i] = (half_t)((float)sum_out[base + i] * r * (float)w[i]);
 }
 
+// Same operation with every element held in registers between the two phases: one 16-byte load of
+// a, b and w per chunk, one global round trip in total.  512 threads, CPT chunks of 8 halves each.
+template <int CPT>
+__global__ void __launch_bounds__(512)
+add_rms_norm_vec_kernel(half_t* sum_out, half_t* norm_out, const half_t* a, const half_t* b, const half_t* w, float eps,
+                        int hidden) {
+    __shared__ float red[8];
+    const size_t base = (size_t)blockIdx.x * hidden;
+    const int chunks = hidden / 8;
+    half8_t va[CPT], vb[CPT], vw[CPT];
+    const half8_t zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+    for (int j = 0; j < CPT; ++j) {
+        const int c = threadIdx.x + j * 512;
+        const bool ok = c < chunks;
+        va[j] = ok ? reinterpret_cast<const half8_t*>(a + base)[c] : zero8;
+        vb[j] = ok ? reinterpret_cast<const half8_t*>(b + base)[c] : zero8;
+        vw[j] = ok ? reinterpret_cast<const half8_t*>(w)[c] : zero8;
+    }
+    float ss = 0.f;
+#pragma unroll
+    for (int j = 0; j < CPT; ++j)
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const half_t s = (half_t)((float)va[j][i] + (float)vb[j][i]);
+            va[j][i] = s;
+            ss = __builtin_fmaf((float)s, (float)s, ss);
+        }
+    ss += dppf<0xB1>(ss);
+    ss += dppf<0x4E>(ss);
+    ss += dppf<0x141>(ss);
+    ss += dppf<0x140>(ss);
+    ss += __shfl_xor(ss, 16, 64);
+    ss += __shfl_xor(ss, 32, 64);
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = ss;
+    __syncthreads();
+    float total = 0.f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) total += red[i];
+    const float r = 1.0f / sqrtf(total / (float)hidden + eps);
+#pragma unroll
+    for (int j = 0; j < CPT; ++j) {
+        const int c = threadIdx.x + j * 512;
+        if (c < chunks) {
+            half8_t n;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) n[i] = (half_t)((float)va[j][i] * r * (float)vw[j][i]);
+            reinterpret_cast<half8_t*>(sum_out + base)[c] = va[j];
+            reinterpret_cast<half8_t*>(norm_out + base)[c] = n;
+        }
+    }
+}
+
 // Library-owned fp32 workspace for the chunk partials, grown on demand.
 static std::mutex g_ws_mu;
 static float* g_ws = nullptr;
@@ -242,18 +329,18 @@ static int workspace(size_t floats, float** out) {
 
 extern "C" {
 
-int tl_decode_attention_f16(void* out, const void* q, const void* cache_k, const void* cache_v, int T, int n_heads,
-                            int head_dim) {
+static int launch_decode_attention(void* out, const void* q, void* cache_k, void* cache_v, int T, int n_heads,
+                                   int head_dim, bool fuse_rope, const char* name) {
     TL_ENSURE_INIT();
-    TL_REQUIRE(out && q && cache_k && cache_v, "tl_decode_attention_f16: null pointer");
-    TL_REQUIRE(T >= 1 && n_heads >= 1, "tl_decode_attention_f16: bad sizes T=%d n_heads=%d", T, n_heads);
-    TL_REQUIRE(head_dim == 64 || head_dim == 128 || head_dim == 256,
-               "tl_decode_attention_f16: head_dim %d not supported (64, 128 or 256)", head_dim);
+    TL_REQUIRE(out && q && cache_k && cache_v, "%s: null pointer", name);
+    TL_REQUIRE(T >= 1 && n_heads >= 1, "%s: bad sizes T=%d n_heads=%d", name, T, n_heads);
+    TL_REQUIRE(head_dim == 64 || head_dim == 128 || head_dim == 256, "%s: head_dim %d not supported (64, 128 or 256)",
+               name, head_dim);
     TL_REQUIRE(tl::aligned16(q) && tl::aligned16(cache_k) && tl::aligned16(cache_v),
-               "tl_decode_attention_f16: q and the caches must be 16-byte aligned");
-    TL_REQUIRE(n_heads <= 65535, "tl_decode_attention_f16: too many heads");
+               "%s: q and the caches must be 16-byte aligned", name);
+    TL_REQUIRE(n_heads <= 65535, "%s: too many heads", name);
     const int n_chunks = (T + tl::kAttnChunk - 1) / tl::kAttnChunk;
-    TL_REQUIRE(n_chunks <= 65535, "tl_decode_attention_f16: T=%d too long", T);
+    TL_REQUIRE(n_chunks <= 65535, "%s: T=%d too long", name, T);
     float* ws = nullptr;
     if (n_chunks > 1) {
         int rc = tl::workspace((size_t)n_heads * n_chunks * (head_dim + 2), &ws);
@@ -264,18 +351,19 @@ int tl_decode_attention_f16(void* out, const void* q, const void* cache_k, const
     const float inv_scale = 1.0f / scale;
     dim3 grid(n_heads, n_chunks);
     hipStream_t st = tl::stream();
-    if (head_dim == 64)
-        hipLaunchKernelGGL(tl::decode_attn_partial_kernel<8>, grid, dim3(tl::kAttnThreads), 0, st, (tl::half_t*)out, ws,
-                           (const tl::half_t*)q, (const tl::half_t*)cache_k, (const tl::half_t*)cache_v, T, n_heads,
-                           inv_scale, n_chunks);
-    else if (head_dim == 128)
-        hipLaunchKernelGGL(tl::decode_attn_partial_kernel<16>, grid, dim3(tl::kAttnThreads), 0, st, (tl::half_t*)out,
-                           ws, (const tl::half_t*)q, (const tl::half_t*)cache_k, (const tl::half_t*)cache_v, T, n_heads,
-                           inv_scale, n_chunks);
-    else
-        hipLaunchKernelGGL(tl::decode_attn_partial_kernel<32>, grid, dim3(tl::kAttnThreads), 0, st, (tl::half_t*)out,
-                           ws, (const tl::half_t*)q, (const tl::half_t*)cache_k, (const tl::half_t*)cache_v, T, n_heads,
-                           inv_scale, n_chunks);
+    auto launch = [&](auto kernel) {
+        hipLaunchKernelGGL(kernel, grid, dim3(tl::kAttnThreads), 0, st, (tl::half_t*)out, ws, (const tl::half_t*)q,
+                           (tl::half_t*)cache_k, (tl::half_t*)cache_v, T, n_heads, inv_scale, n_chunks);
+    };
+    if (fuse_rope) {
+        if (head_dim == 64) launch(tl::decode_attn_partial_kernel<8, true>);
+        else if (head_dim == 128) launch(tl::decode_attn_partial_kernel<16, true>);
+        else launch(tl::decode_attn_partial_kernel<32, true>);
+    } else {
+        if (head_dim == 64) launch(tl::decode_attn_partial_kernel<8, false>);
+        else if (head_dim == 128) launch(tl::decode_attn_partial_kernel<16, false>);
+        else launch(tl::decode_attn_partial_kernel<32, false>);
+    }
     TL_CHECK_LAUNCH("decode_attn_partial_kernel");
     if (n_chunks > 1) {
         hipLaunchKernelGGL(tl::decode_attn_merge_kernel, dim3(n_heads), dim3(256), 0, st, (tl::half_t*)out, ws, head_dim,
@@ -283,6 +371,19 @@ int tl_decode_attention_f16(void* out, const void* q, const void* cache_k, const
         TL_CHECK_LAUNCH("decode_attn_merge_kernel");
     }
     return TL_OK;
+}
+
+int tl_decode_attention_f16(void* out, const void* q, const void* cache_k, const void* cache_v, int T, int n_heads,
+                            int head_dim) {
+    return launch_decode_attention(out, q, const_cast<void*>(cache_k), const_cast<void*>(cache_v), T, n_heads, head_dim,
+                                   false, "tl_decode_attention_f16");
+}
+
+int tl_decode_attention_rope_f16(void* out, const void* qkv, void* cache_k, void* cache_v, int pos, int n_heads,
+                                 int head_dim) {
+    TL_REQUIRE(pos >= 0, "tl_decode_attention_rope_f16: negative position");
+    return launch_decode_attention(out, qkv, cache_k, cache_v, pos + 1, n_heads, head_dim, true,
+                                   "tl_decode_attention_rope_f16");
 }
 
 int tl_rope_qk_store_kv_f16(void* qkv, void* cache_k, void* cache_v, int pos, int n_heads, int head_dim) {
@@ -305,9 +406,23 @@ int tl_add_rms_norm_f16(void* sum_out, void* norm_out, const void* a, const void
     TL_REQUIRE(sum_out && norm_out && a && b && weight, "tl_add_rms_norm_f16: null pointer");
     TL_REQUIRE(hidden_size > 0 && num_tokens >= 0, "tl_add_rms_norm_f16: bad sizes");
     if (num_tokens == 0) return TL_OK;
-    hipLaunchKernelGGL(tl::add_rms_norm_kernel, dim3(num_tokens), dim3(256), 0, tl::stream(), (tl::half_t*)sum_out,
-                       (tl::half_t*)norm_out, (const tl::half_t*)a, (const tl::half_t*)b, (const tl::half_t*)weight,
-                       eps, hidden_size);
+    const bool vec = hidden_size % 8 == 0 && hidden_size <= 512 * 8 * 4 && tl::aligned16(sum_out) &&
+                     tl::aligned16(norm_out) && tl::aligned16(a) && tl::aligned16(b) && tl::aligned16(weight);
+    if (vec) {
+        const int cpt = (hidden_size / 8 + 511) / 512;
+        auto launch = [&](auto kernel) {
+            hipLaunchKernelGGL(kernel, dim3(num_tokens), dim3(512), 0, tl::stream(), (tl::half_t*)sum_out,
+                               (tl::half_t*)norm_out, (const tl::half_t*)a, (const tl::half_t*)b,
+                               (const tl::half_t*)weight, eps, hidden_size);
+        };
+        if (cpt <= 1) launch(tl::add_rms_norm_vec_kernel<1>);
+        else if (cpt == 2) launch(tl::add_rms_norm_vec_kernel<2>);
+        else launch(tl::add_rms_norm_vec_kernel<4>);
+    } else {
+        hipLaunchKernelGGL(tl::add_rms_norm_kernel, dim3(num_tokens), dim3(256), 0, tl::stream(), (tl::half_t*)sum_out,
+                           (tl::half_t*)norm_out, (const tl::half_t*)a, (const tl::half_t*)b,
+                           (const tl::half_t*)weight, eps, hidden_size);
+    }
     TL_CHECK_LAUNCH("add_rms_norm_kernel");
     return TL_OK;
 }

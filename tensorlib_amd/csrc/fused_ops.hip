@@ -299,17 +299,31 @@ static int launch_strided(void* dense, void* base, const int* shape, const int* 
 
 // One workgroup per row; ties resolve to the smallest index (the CPU backend's strict '>',
 // tensorLib/src/device/cpu/CPU.cpp:356-372).  A row with no element above -inf returns 0.
-__global__ void __launch_bounds__(256)
+template <bool VEC>
+__global__ void __launch_bounds__(1024)
 argmax_kernel(int* out, const half_t* in, size_t reduce_size) {
-    __shared__ float sv[256];
-    __shared__ int si[256];
+    __shared__ float sv[1024];
+    __shared__ int si[1024];
     constexpr int kNone = 0x7fffffff;
     const half_t* x = in + (size_t)blockIdx.x * reduce_size;
     float best = -INFINITY;
     int bi = kNone;
-    for (size_t j = threadIdx.x; j < reduce_size; j += blockDim.x) {
-        const float v = (float)x[j];
-        if (v > best) { best = v; bi = (int)j; }
+    if constexpr (VEC) {
+        // 16-byte loads; a thread visits its chunks, and the elements of a chunk, in increasing index order
+        const size_t chunks = reduce_size / 8;
+        for (size_t c = threadIdx.x; c < chunks; c += blockDim.x) {
+            const half8_t v8 = reinterpret_cast<const half8_t*>(x)[c];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const float v = (float)v8[e];
+                if (v > best) { best = v; bi = (int)(c * 8 + e); }
+            }
+        }
+    } else {
+        for (size_t j = threadIdx.x; j < reduce_size; j += blockDim.x) {
+            const float v = (float)x[j];
+            if (v > best) { best = v; bi = (int)j; }
+        }
     }
     sv[threadIdx.x] = best;
     si[threadIdx.x] = bi;
@@ -454,7 +468,13 @@ int tl_argmax_f16(int* out, const void* in, size_t reduce_size, size_t num_eleme
     const size_t rows = num_elements / reduce_size;
     if (rows == 0) return TL_OK;
     TL_REQUIRE(rows <= 0x7fffffffu && reduce_size <= 0x7fffffffu, "tl_argmax_f16: size out of range");
-    hipLaunchKernelGGL(tl::argmax_kernel, dim3((unsigned)rows), dim3(256), 0, tl::stream(), out,
+    const bool vec = reduce_size % 8 == 0 && tl::aligned16(in);
+    const int threads = reduce_size >= 8192 ? 1024 : 256;
+    if (vec)
+        hipLaunchKernelGGL(tl::argmax_kernel<true>, dim3((unsigned)rows), dim3(threads), 0, tl::stream(), out,
+                           (const tl::half_t*)in, reduce_size);
+    else
+        hipLaunchKernelGGL(tl::argmax_kernel<false>, dim3((unsigned)rows), dim3(threads), 0, tl::stream(), out,
                        (const tl::half_t*)in, reduce_size);
     TL_CHECK_LAUNCH("argmax_kernel");
     return TL_OK;

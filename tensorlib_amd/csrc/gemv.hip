@@ -191,6 +191,7 @@ __global__ void __launch_bounds__(WAVES * 64) gemv_f16_wave_kernel(GemvArgs a) {
 //   XMODE 0: x goes global -> LDS (whole vector, once per workgroup) -> registers;
 //            the first W tile is requested before the staging barrier.
 //   XMODE 1: every wavefront reads its own K segment of x straight into registers.
+//   XMODE 2: like 1, but x is silu(a) * b of a [a | b] input (the SwiGLU gate fused into the load).
 // Dynamic LDS: [K8 chunks of x when XMODE == 0] + 2*RG*KSPLIT*ROWS floats when KSPLIT > 1.
 template <int WAVES, int ROWS, int UNROLL, int KSPLIT, int XMODE>
 __global__ void __launch_bounds__(WAVES * 64) gemv_f16_stream_kernel(GemvArgs a) {
@@ -228,6 +229,20 @@ __global__ void __launch_bounds__(WAVES * 64) gemv_f16_stream_kernel(GemvArgs a)
     if constexpr (XMODE == 1) {
 #pragma unroll
         for (int u = 0; u < UNROLL; ++u) xv[u] = ok[u] ? x[cidx[u]] : zero8;
+    }
+    if constexpr (XMODE == 2) {
+        // x is given as [a | b] (2*K halves); the vector that is multiplied is silu(a) * b, computed in
+        // fp32 and rounded to fp16 once, exactly what tl_silu_mul_f16 would have written to memory
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u) {
+            const half8_t va = ok[u] ? x[cidx[u]] : zero8;
+            const half8_t vb = ok[u] ? x[K8 + cidx[u]] : zero8;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const float a = (float)va[i];
+                xv[u][i] = (half_t)(a * (1.0f / (1.0f + expf(-a))) * (float)vb[i]);
+            }
+        }
     }
 
     half8_t cur[ROWS][UNROLL], nxt[ROWS][UNROLL];
@@ -392,6 +407,8 @@ static const GemvVariant g_variants[] = {
     TL_STREAM2(8, 1, 6, 4),       // 45, 46
     TL_STREAM2(4, 1, 6, 4),       // 47, 48
     TL_STREAM2(4, 1, 2, 4),       // 49, 50
+    TL_STREAM(4, 2, 2, 4, 2),     // 51  silu*mul prologue, K <= 4096
+    TL_STREAM(8, 2, 3, 8, 2),     // 52  silu*mul prologue, K <= 12288
 };
 static constexpr int kNumVariants = sizeof(g_variants) / sizeof(g_variants[0]);
 static int g_forced_variant = 0;
@@ -425,7 +442,7 @@ static int pick_variant(size_t N, size_t K, int* waves_per_cu) {
 }
 
 int launch_gemv(const void* x, const void* W, void* y, size_t N, size_t K, size_t batch, size_t sx,
-                size_t sw, size_t sy) {
+                size_t sw, size_t sy, int prologue) {
     if (N == 0 || batch == 0) return TL_OK;
     TL_REQUIRE(N <= 0x7fffffffu && K <= 0x7fffffffu && batch <= 65535, "gemv: size out of range");
     const DeviceInfo& dev = device_info();
@@ -479,6 +496,15 @@ int launch_gemv(const void* x, const void* W, void* y, size_t N, size_t K, size_
 
     int auto_wpc = 16;
     int vi = g_forced_variant ? g_forced_variant : pick_variant(N, K, &auto_wpc);
+    if (prologue == 1) {
+        static const int v_k4096 = variant_index("stream_w4r2u2s4x2");
+        static const int v_k12288 = variant_index("stream_w8r2u3s8x2");
+        if (a.K8 <= 512) { vi = v_k4096; auto_wpc = 1 << 20; }
+        else if (a.K8 <= 1536) { vi = v_k12288; auto_wpc = 16; }
+        else return set_error(TL_ELIMIT, "gemv with fused silu*mul: K=%zu exceeds 12288", K);
+    }
+    TL_REQUIRE(g_variants[vi].xmode != 2 || prologue == 1,
+               "gemv variant %s cannot hold a plain x: it reads an [a | b] input of 2*K halves", g_variants[vi].name);
     if (g_variants[vi].xmode >= 0) {
         // the streaming kernel needs a wavefront's K segment to fit one register tile
         const GemvVariant& sv = g_variants[vi];
@@ -493,7 +519,7 @@ int launch_gemv(const void* x, const void* W, void* y, size_t N, size_t K, size_
     const int rg = v.waves / v.ksplit;
     const int rows_per_block = rg * v.rows;
     a.num_row_blocks = (int)((N + rows_per_block - 1) / rows_per_block);
-    size_t lds = (v.xmode == 1 ? 0 : (size_t)a.K8 * 16) +
+    size_t lds = (v.xmode >= 1 ? 0 : (size_t)a.K8 * 16) +
                  (v.ksplit > 1 ? (size_t)(v.xmode >= 0 ? 2 : 1) * rg * v.ksplit * v.rows * 4 : 0);
     if (lds > 64 * 1024) {
         // x does not fit the default LDS window: fall back to the generic kernel.
@@ -523,7 +549,7 @@ extern "C" {
 int tl_gemv_f16(const void* x, const void* W, void* y, size_t N, size_t K) {
     TL_ENSURE_INIT();
     TL_REQUIRE(x && W && y, "tl_gemv_f16: null pointer");
-    return tl::launch_gemv(x, W, y, N, K, 1, 0, 0, 0);
+    return tl::launch_gemv(x, W, y, N, K, 1, 0, 0, 0, 0);
 }
 
 int tl_set_gemv_variant(int variant) {
@@ -544,3 +570,12 @@ int tl_set_gemv_grid_waves_per_cu(int waves) {
 }
 
 }  // extern "C"
+
+extern "C" int tl_gemv_silu_mul_f16(const void* ab, const void* W, void* y, size_t N, size_t K) {
+    TL_ENSURE_INIT();
+    TL_REQUIRE(ab && W && y, "tl_gemv_silu_mul_f16: null pointer");
+    TL_REQUIRE(K % 8 == 0 && tl::aligned16(ab) && tl::aligned16(W),
+               "tl_gemv_silu_mul_f16: needs K %% 8 == 0 and 16-byte aligned operands");
+    TL_REQUIRE(K / 8 >= 64, "tl_gemv_silu_mul_f16: K=%zu too short for the fused kernel (K >= 512)", K);
+    return tl::launch_gemv(ab, W, y, N, K, 1, 0, 0, 0, 1);
+}

@@ -664,7 +664,7 @@ int tl_hgemm_f16(const void* A, const void* B, void* C, size_t M, size_t N, size
 int tl_matmul2d_f16(const void* A, const void* B, void* C, size_t M, size_t N, size_t K) {
     TL_ENSURE_INIT();
     TL_REQUIRE(A && B && C, "tl_matmul2d_f16: null pointer");
-    if (M == 1) return tl::launch_gemv(A, B, C, N, K, 1, 0, 0, 0);
+    if (M == 1) return tl::launch_gemv(A, B, C, N, K, 1, 0, 0, 0, 0);
     return tl::launch_hgemm(A, B, C, M, N, K, 1, 0, 0, 0);
 }
 
@@ -673,7 +673,7 @@ int tl_matmul2d_batched_f16(const void* A, const void* B, void* C, size_t M, siz
     TL_ENSURE_INIT();
     TL_REQUIRE(A && B && C, "tl_matmul2d_batched_f16: null pointer");
     TL_REQUIRE(batch <= 65535, "tl_matmul2d_batched_f16: batch %zu exceeds 65535", batch);
-    if (M == 1) return tl::launch_gemv(A, B, C, N, K, batch, strideA, strideB, strideC);
+    if (M == 1) return tl::launch_gemv(A, B, C, N, K, batch, strideA, strideB, strideC, 0);
     return tl::launch_hgemm(A, B, C, M, N, K, batch, strideA, strideB, strideC);
 }
 

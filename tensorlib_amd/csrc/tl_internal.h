@@ -42,7 +42,7 @@ int launch_fill_f16(void* out, uint16_t bits, size_t n);
 
 // Shared launchers (batch strides in elements; batch == 1 ignores them).
 int launch_gemv(const void* x, const void* W, void* y, size_t N, size_t K, size_t batch, size_t sx,
-                size_t sw, size_t sy);
+                size_t sw, size_t sy, int prologue);
 int launch_hgemm(const void* A, const void* B, void* C, size_t M, size_t N, size_t K, size_t batch,
                  size_t sa, size_t sb, size_t sc);
 

@@ -292,6 +292,43 @@ class HipDevice:
               "tl_decode_attention_f16")
         return out
 
+    def decode_attention_rope(self, qkv: torch.Tensor, cache_k: torch.Tensor, cache_v: torch.Tensor, pos: int):
+        """qkv: [3, n_heads, head_dim] raw projections of the token at `pos`; writes cache rows `pos`."""
+        _req(qkv, name="qkv"), _req(cache_k, name="cache_k"), _req(cache_v, name="cache_v")
+        _, H, D = qkv.shape
+        if cache_k.shape[1:] != (H, D) or cache_v.shape != cache_k.shape or pos >= cache_k.shape[0]:
+            raise ValueError("cache shape does not match qkv / pos")
+        out = self.empty(H, D)
+        check(self.lib.tl_decode_attention_rope_f16(_ptr(out), _ptr(qkv), _ptr(cache_k), _ptr(cache_v), pos, H, D),
+              "tl_decode_attention_rope_f16")
+        return out
+
+    def rope_qk_store_kv(self, qkv: torch.Tensor, cache_k: torch.Tensor, cache_v: torch.Tensor, pos: int):
+        _req(qkv, name="qkv"), _req(cache_k, name="cache_k"), _req(cache_v, name="cache_v")
+        _, H, D = qkv.shape
+        check(self.lib.tl_rope_qk_store_kv_f16(_ptr(qkv), _ptr(cache_k), _ptr(cache_v), pos, H, D),
+              "tl_rope_qk_store_kv_f16")
+
+    def add_rms_norm(self, a: torch.Tensor, b: torch.Tensor, weight: torch.Tensor, eps: float, sum_out=None, norm_out=None):
+        _req(a, name="a"), _req(b, name="b"), _req(weight, name="weight")
+        hidden = a.shape[-1]
+        tokens = a.numel() // hidden
+        sum_out = torch.empty_like(a) if sum_out is None else sum_out
+        norm_out = torch.empty_like(a) if norm_out is None else norm_out
+        check(self.lib.tl_add_rms_norm_f16(_ptr(sum_out), _ptr(norm_out), _ptr(a), _ptr(b), _ptr(weight), eps, hidden,
+                                           tokens), "tl_add_rms_norm_f16")
+        return sum_out, norm_out
+
+    def gemv_silu_mul(self, ab: torch.Tensor, W: torch.Tensor) -> torch.Tensor:
+        """y = W . (silu(ab[:K]) * ab[K:]) with W [N, K] and ab of 2*K halves."""
+        _req(ab, name="ab"), _req(W, name="W")
+        N, K = W.shape
+        if ab.numel() != 2 * K:
+            raise ValueError("ab must hold 2*K elements")
+        y = self.empty(N)
+        check(self.lib.tl_gemv_silu_mul_f16(_ptr(ab), _ptr(W), _ptr(y), N, K), "tl_gemv_silu_mul_f16")
+        return y
+
     # -- tuning hooks -------------------------------------------------------------------
     def set_gemv_variant(self, v: int) -> None:
         check(self.lib.tl_set_gemv_variant(v), "tl_set_gemv_variant")

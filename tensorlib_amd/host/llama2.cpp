@@ -178,8 +178,8 @@ struct tlm_model {
                 gemv(x_norm.p, w.wk, xk(1), dim, dim);
                 gemv(x_norm.p, w.wv, xv(1), dim, dim);
             }
-            ck(tl_rope_qk_store_kv_f16(qkv.p, cache_k[l].p, cache_v[l].p, pos, H, D), "rope_qk_store_kv");
-            ck(tl_decode_attention_f16(o_c.p, qkv.p, cache_k[l].p, cache_v[l].p, pos + 1, H, D), "decode_attention");
+            // RoPE(q), RoPE(k) -> cache_k[pos], v -> cache_v[pos] and the attention itself, cache read in place
+            ck(tl_decode_attention_rope_f16(o_c.p, qkv.p, cache_k[l].p, cache_v[l].p, pos, H, D), "decode_attention_rope");
             gemv(o_c.p, w.wo, x_norm.p, dim, dim);
             // h = x + attn ; x_norm = rmsnorm(h) * ffn_norm
             ck(tl_add_rms_norm_f16(x_residual.p, x_norm.p, x.p, x_norm.p, w.ffn_norm, eps, dim, 1), "add_rms_norm");
@@ -189,8 +189,13 @@ struct tlm_model {
                 gemv(x_norm.p, w.w1, x1(1), hidden, dim);
                 gemv(x_norm.p, w.w3, x3(1), hidden, dim);
             }
-            ck(tl_silu_mul_f16(x2.p, x1(1), x3(1), hidden), "silu_mul");
-            gemv(x2.p, w.w2, x.p, dim, hidden);
+            if (hidden % 8 == 0 && hidden >= 512 && hidden <= 12288) {
+                // silu(x1) * x3 is formed while w2's GEMV loads its input
+                ck(tl_gemv_silu_mul_f16(x13.p, w.w2, x.p, dim, hidden), "gemv_silu_mul");
+            } else {
+                ck(tl_silu_mul_f16(x2.p, x1(1), x3(1), hidden), "silu_mul");
+                gemv(x2.p, w.w2, x.p, dim, hidden);
+            }
             // x = h + ffn ; x_norm = rmsnorm(x) * (next layer's attention norm | final norm)
             const half* next_norm = (l + 1 < n_layers) ? layers[l + 1].att_norm : final_norm;
             ck(tl_add_rms_norm_f16(x.p, x_norm.p, x_residual.p, x.p, next_norm, eps, dim, 1), "add_rms_norm");

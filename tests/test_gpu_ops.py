@@ -7,7 +7,7 @@ import pytest
 import torch
 
 from tensorlib_amd import synth
-from tests.conftest import assert_close_f16
+from tests.conftest import assert_close_f16, assert_close_scaled
 
 pytestmark = pytest.mark.gpu
 RTOL, ATOL = 1e-2, 1e-3
@@ -188,3 +188,87 @@ def test_decode_attention_fused_vs_chain(dev, oracle, T, H, D):
     got = dev.decode_attention(dev.from_numpy(q), dev.from_numpy(ck), dev.from_numpy(cv), T).cpu().numpy()
     want = _attention_chain_oracle(oracle, q, ck, cv, T)
     assert_close_f16(got, want, RTOL, 2e-3, f"decode attention T={T}")
+
+
+@pytest.mark.parametrize("tokens,hidden", [(1, 4096), (3, 264), (2, 100), (1, 11008), (5, 16384), (1, 20000)])
+def test_add_rms_norm(dev, oracle, tokens, hidden):
+    """EwiseAdd followed by RMSNorm in one launch; also with the aliasing the driver uses."""
+    a = synth.normal_f16(100, (tokens, hidden), 1.0)
+    b = synth.normal_f16(101, (tokens, hidden), 1.5)
+    w = synth.normal_f16(102, (hidden,), 1.0)
+    want_sum = oracle.binary(a, b, "add")
+    want_norm = oracle.rms_norm(want_sum, w, 1e-5, "exact")
+    s, n = dev.add_rms_norm(dev.from_numpy(a), dev.from_numpy(b), dev.from_numpy(w), 1e-5)
+    assert np.array_equal(s.cpu().numpy().view(np.uint16), want_sum.view(np.uint16))
+    assert_close_f16(n.cpu().numpy(), want_norm, RTOL, ATOL, "add_rms_norm")
+    ad, bd = dev.from_numpy(a), dev.from_numpy(b)
+    dev.add_rms_norm(ad, bd, dev.from_numpy(w), 1e-5, sum_out=ad, norm_out=bd)   # sum over a, norm over b
+    assert np.array_equal(ad.cpu().numpy().view(np.uint16), want_sum.view(np.uint16))
+    assert_close_f16(bd.cpu().numpy(), want_norm, RTOL, ATOL, "add_rms_norm aliased")
+
+
+@pytest.mark.parametrize("H,D,pos", [(32, 128, 0), (32, 128, 1023), (4, 64, 17), (2, 256, 5)])
+def test_rope_qk_store_kv(dev, oracle, H, D, pos):
+    S = pos + 3
+    qkv = synth.normal_f16(110, (3, H, D), 1.0)
+    ck0 = synth.normal_f16(111, (S, H, D), 1.0)
+    cv0 = synth.normal_f16(112, (S, H, D), 1.0)
+    qd, kd, vd = dev.from_numpy(qkv), dev.from_numpy(ck0), dev.from_numpy(cv0)
+    dev.rope_qk_store_kv(qd, kd, vd, pos)
+    q_want = oracle.rope(qkv[0].reshape(1, 1, H, D), pos).reshape(H, D)
+    k_want = oracle.rope(qkv[1].reshape(1, 1, H, D), pos).reshape(H, D)
+    got = qd.cpu().numpy()
+    assert_close_f16(got[0], q_want, RTOL, 2e-3, "q rope")
+    assert np.array_equal(got[1:].view(np.uint16), qkv[1:].view(np.uint16))      # k, v inputs untouched
+    ck, cv = kd.cpu().numpy(), vd.cpu().numpy()
+    assert_close_f16(ck[pos], k_want, RTOL, 2e-3, "k rope into cache")
+    assert np.array_equal(cv[pos].view(np.uint16), qkv[2].view(np.uint16))
+    keep = np.arange(S) != pos
+    assert np.array_equal(ck[keep].view(np.uint16), ck0[keep].view(np.uint16))
+    assert np.array_equal(cv[keep].view(np.uint16), cv0[keep].view(np.uint16))
+
+
+@pytest.mark.parametrize("pos,H,D", [(0, 32, 128), (63, 32, 128), (64, 32, 128), (1023, 32, 128), (100, 4, 64), (70, 2, 256)])
+def test_decode_attention_rope_equals_separate_steps(dev, oracle, pos, H, D):
+    """The fused launch must give exactly what rope_qk_store_kv followed by decode_attention gives,
+    and leave the caches in the same state."""
+    S = pos + 2
+    qkv = synth.normal_f16(120, (3, H, D), 1.0)
+    ck0 = synth.normal_f16(121, (S, H, D), 1.0)
+    cv0 = synth.normal_f16(122, (S, H, D), 1.0)
+    q1, k1, v1 = dev.from_numpy(qkv), dev.from_numpy(ck0), dev.from_numpy(cv0)
+    dev.rope_qk_store_kv(q1, k1, v1, pos)
+    want = dev.decode_attention(q1[0].contiguous(), k1, v1, pos + 1).cpu().numpy()
+    q2, k2, v2 = dev.from_numpy(qkv), dev.from_numpy(ck0), dev.from_numpy(cv0)
+    got = dev.decode_attention_rope(q2, k2, v2, pos).cpu().numpy()
+    assert np.array_equal(got.view(np.uint16), want.view(np.uint16))
+    assert torch.equal(k1, k2) and torch.equal(v1, v2)
+    assert np.array_equal(q2.cpu().numpy().view(np.uint16), qkv.view(np.uint16))   # raw projections untouched
+    # and against the CPU chain
+    q_rot = oracle.rope(qkv[0].reshape(1, 1, H, D), pos).reshape(H, D)
+    ck = ck0.copy(); cv = cv0.copy()
+    ck[pos] = oracle.rope(qkv[1].reshape(1, 1, H, D), pos).reshape(H, D)
+    cv[pos] = qkv[2]
+    assert_close_f16(got, _attention_chain_oracle(oracle, q_rot, ck, cv, pos + 1), RTOL, 2e-3, "fused rope attention")
+
+
+@pytest.mark.parametrize("N,K", [(4096, 11008), (300, 512), (64, 4096), (33, 12288), (10, 520)])
+def test_gemv_silu_mul(dev, oracle, N, K):
+    ab = synth.normal_f16(130, (2 * K,), 1.5)
+    W = synth.normal_f16(131, (N, K), 0.02)
+    got = dev.gemv_silu_mul(dev.from_numpy(ab), dev.from_numpy(W)).cpu().numpy()
+    x2 = oracle.silu_mul(ab[:K], ab[K:])
+    # silu*mul is rounded once on the GPU and twice on the CPU chain: compare on the output scale
+    assert_close_scaled(got, oracle.matmul2d(x2[None, :], W)[0], 1e-2, 5e-3, "gemv with fused silu*mul")
+    # identical bits to the two-step GPU path
+    x2d = dev.silu_mul(dev.from_numpy(ab[:K]), dev.from_numpy(ab[K:]))
+    two = dev.gemv(x2d, dev.from_numpy(W)).cpu().numpy()
+    assert np.array_equal(got.view(np.uint16), two.view(np.uint16))
+
+
+def test_gemv_silu_mul_limits(dev):
+    from tensorlib_amd import TensorLibError
+    with pytest.raises(TensorLibError):
+        dev.gemv_silu_mul(dev.empty(2 * 16384), dev.empty(8, 16384))     # K beyond the fused kernel's limit
+    with pytest.raises(TensorLibError):
+        dev.gemv_silu_mul(dev.empty(2 * 100), dev.empty(8, 100))         # K not a multiple of 8
