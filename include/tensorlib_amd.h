@@ -188,9 +188,16 @@ int tl_gemv_silu_mul_f16(const void* ab, const void* W, void* y, size_t N, size_
 
 /* tl_rope_qk_store_kv_f16 + tl_decode_attention_f16 in one launch pair: qkv is the raw q|k|v
  * projection of the token at position `pos`; q is rotated on load, the rotated k and the v row
- * are written to cache_k[pos] / cache_v[pos], and out[h,:] attends to positions 0..pos. */
-int tl_decode_attention_rope_f16(void* out, const void* qkv, void* cache_k, void* cache_v, int pos,
-                                 int n_heads, int head_dim);
+ * are written to cache_k[pos] / cache_v[pos], and out[h,:] attends to positions 0..pos.
+ * rope_table: NULL, or a table from tl_rope_table_f16 covering `pos` (saves the sin/cos/pow). */
+int tl_decode_attention_rope_f16(void* out, const void* qkv, void* cache_k, void* cache_v,
+                                 const void* rope_table, int pos, int n_heads, int head_dim);
+
+/* table[pos][pair] = (half(cos), half(sin)) of pos / 10000^(2*pair/head_dim) for pos < max_seq:
+ * max_seq * head_dim halves.  The same values every RoPE entry point computes on the fly
+ * (tensorLib/src/device/cpu/CPU.cpp:444-447); the reference's own precompute_freqs table is unused
+ * (model/llama2_7b/src/Transformer.cpp:203-216). */
+int tl_rope_table_f16(void* table, int max_seq, int head_dim);
 
 /* Decode-step glue after a fused q|k|v projection (qkv = [q | k | v], each n_heads*head_dim
  * halves): rotary-embed q in place, rotary-embed k into cache_k[pos], copy v into cache_v[pos]

@@ -54,13 +54,39 @@ __device__ __forceinline__ half8_t rope_chunk(half8_t v, int pos, int d0, int he
     return r;
 }
 
+// Same rotation with (cos, sin) pairs read from a table built by rope_table_kernel.
+__device__ __forceinline__ half8_t rope_chunk_cs(half8_t v, half8_t cs) {
+    half8_t r;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const float c = (float)cs[2 * i], s = (float)cs[2 * i + 1];
+        const float v0 = (float)v[2 * i], v1 = (float)v[2 * i + 1];
+        r[2 * i] = (half_t)(v0 * c - v1 * s);
+        r[2 * i + 1] = (half_t)(v0 * s + v1 * c);
+    }
+    return r;
+}
+
+// table[pos][pair] = (half(cos(theta)), half(sin(theta))), theta = pos / 10000^(2*pair/head_dim) in fp32:
+// the values every RoPE kernel of this library computes on the fly.
+__global__ void __launch_bounds__(256) rope_table_kernel(half_t* table, int max_seq, int head_dim) {
+    const int half_d = head_dim / 2;
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= (size_t)max_seq * half_d) return;
+    const int pos = (int)(i / half_d), pair = (int)(i % half_d);
+    const float theta = (float)pos * 1.0f / powf(10000.0f, (float)(2 * pair) / (float)head_dim);
+    half2_t cs = {(half_t)cosf(theta), (half_t)sinf(theta)};
+    *reinterpret_cast<half2_t*>(table + 2 * i) = cs;
+}
+
 // FUSE_ROPE: `q` points at the raw q|k|v projection of the new token (position T-1).  q is rotated
 // on load; the workgroup that owns the last chunk rotates the new k row, uses it, and writes it and
 // the new v row into the caches (each head's workgroup writes only its own head slice).
 template <int LPR, bool FUSE_ROPE>
 __global__ void __launch_bounds__(kAttnThreads)
 decode_attn_partial_kernel(half_t* out, float* partial, const half_t* q, half_t* cache_k,
-                           half_t* cache_v, int T, int n_heads, float inv_scale, int n_chunks) {
+                           half_t* cache_v, const half_t* rope_table, int T, int n_heads, float inv_scale,
+                           int n_chunks) {
     constexpr int D = LPR * 8;
     constexpr int GROUPS = kAttnThreads / LPR;
     __shared__ float sc[kAttnChunk];
@@ -77,23 +103,55 @@ decode_attn_partial_kernel(half_t* out, float* partial, const half_t* q, half_t*
     const size_t row_stride = (size_t)n_heads * D;
 
     half8_t qv = *reinterpret_cast<const half8_t*>(q + (size_t)h * D + sub * 8);
-    if constexpr (FUSE_ROPE) qv = rope_chunk(qv, T - 1, sub * 8, D);
+    half8_t cs = {0, 0, 0, 0, 0, 0, 0, 0};  // (cos, sin) of the 4 pairs of this thread's chunk at position T-1
+    if constexpr (FUSE_ROPE) {
+        if (rope_table) {
+            cs = *reinterpret_cast<const half8_t*>(rope_table + ((size_t)(T - 1) * (D / 2) + sub * 4) * 2);
+            qv = rope_chunk_cs(qv, cs);
+        } else {
+            qv = rope_chunk(qv, T - 1, sub * 8, D);
+        }
+    }
+
+    // All K and V rows this thread will touch are requested up front (NIT rows each), so the whole
+    // kernel pays one global round trip instead of one per phase.
+    constexpr int NIT = kAttnChunk / GROUPS;
+    half8_t kreg[NIT], vreg[NIT];
+    const half8_t zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+    const size_t head_off = (size_t)h * D + sub * 8;
+#pragma unroll
+    for (int it = 0; it < NIT; ++it) {
+        const int t = t0 + grp + it * GROUPS;
+        if (t < t1) {
+            if (FUSE_ROPE && t == T - 1) {
+                kreg[it] = *reinterpret_cast<const half8_t*>(q + row_stride + head_off);
+                vreg[it] = *reinterpret_cast<const half8_t*>(q + 2 * row_stride + head_off);
+            } else {
+                kreg[it] = *reinterpret_cast<const half8_t*>(cache_k + (size_t)t * row_stride + head_off);
+                vreg[it] = *reinterpret_cast<const half8_t*>(cache_v + (size_t)t * row_stride + head_off);
+            }
+        } else {
+            kreg[it] = zero8;
+            vreg[it] = zero8;
+        }
+    }
 
     // scores
-    for (int t = t0 + grp; t < t1; t += GROUPS) {
-        half8_t kv;
-        if (FUSE_ROPE && t == T - 1) {
-            kv = *reinterpret_cast<const half8_t*>(q + row_stride + (size_t)h * D + sub * 8);
-            kv = rope_chunk(kv, T - 1, sub * 8, D);
-            *reinterpret_cast<half8_t*>(cache_k + (size_t)t * row_stride + (size_t)h * D + sub * 8) = kv;
-        } else {
-            kv = *reinterpret_cast<const half8_t*>(cache_k + (size_t)t * row_stride + (size_t)h * D + sub * 8);
-        }
-        float s = 0.f;
 #pragma unroll
-        for (int i = 0; i < 8; ++i) s = __builtin_fmaf((float)qv[i], (float)kv[i], s);
-        s = lanes_sum<LPR>(s);
-        if (sub == 0) sc[t - t0] = s * inv_scale;
+    for (int it = 0; it < NIT; ++it) {
+        const int t = t0 + grp + it * GROUPS;
+        if (t < t1) {
+            if (FUSE_ROPE && t == T - 1) {
+                kreg[it] = rope_table ? rope_chunk_cs(kreg[it], cs) : rope_chunk(kreg[it], T - 1, sub * 8, D);
+                *reinterpret_cast<half8_t*>(cache_k + (size_t)t * row_stride + head_off) = kreg[it];
+                *reinterpret_cast<half8_t*>(cache_v + (size_t)t * row_stride + head_off) = vreg[it];
+            }
+            float s = 0.f;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) s = __builtin_fmaf((float)qv[i], (float)kreg[it][i], s);
+            s = lanes_sum<LPR>(s);
+            if (sub == 0) sc[t - t0] = s * inv_scale;
+        }
     }
     __syncthreads();
 
@@ -130,17 +188,14 @@ decode_attn_partial_kernel(half_t* out, float* partial, const half_t* q, half_t*
     float acc[8];
 #pragma unroll
     for (int i = 0; i < 8; ++i) acc[i] = 0.f;
-    for (int t = t0 + grp; t < t1; t += GROUPS) {
-        half8_t vv;
-        if (FUSE_ROPE && t == T - 1) {
-            vv = *reinterpret_cast<const half8_t*>(q + 2 * row_stride + (size_t)h * D + sub * 8);
-            *reinterpret_cast<half8_t*>(cache_v + (size_t)t * row_stride + (size_t)h * D + sub * 8) = vv;
-        } else {
-            vv = *reinterpret_cast<const half8_t*>(cache_v + (size_t)t * row_stride + (size_t)h * D + sub * 8);
-        }
-        const float p = sc[t - t0];
 #pragma unroll
-        for (int i = 0; i < 8; ++i) acc[i] = __builtin_fmaf(p, (float)vv[i], acc[i]);
+    for (int it = 0; it < NIT; ++it) {
+        const int t = t0 + grp + it * GROUPS;
+        if (t < t1) {
+            const float p = sc[t - t0];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) acc[i] = __builtin_fmaf(p, (float)vreg[it][i], acc[i]);
+        }
     }
 #pragma unroll
     for (int i = 0; i < 8; ++i) obuf[grp][sub * 8 + i] = acc[i];
@@ -159,6 +214,9 @@ decode_attn_partial_kernel(half_t* out, float* partial, const half_t* q, half_t*
     }
 }
 
+// Second pass: merge the chunk partials of one head.  (Folding this into the first launch with a
+// "last workgroup merges" ticket was measured slower: the device-scope fences it needs cost more
+// than this 4 us launch.)
 __global__ void __launch_bounds__(256)
 decode_attn_merge_kernel(half_t* out, const float* partial, int D, int n_chunks) {
     const int h = blockIdx.x;
@@ -329,8 +387,8 @@ static int workspace(size_t floats, float** out) {
 
 extern "C" {
 
-static int launch_decode_attention(void* out, const void* q, void* cache_k, void* cache_v, int T, int n_heads,
-                                   int head_dim, bool fuse_rope, const char* name) {
+static int launch_decode_attention(void* out, const void* q, void* cache_k, void* cache_v, const void* rope_table,
+                                   int T, int n_heads, int head_dim, bool fuse_rope, const char* name) {
     TL_ENSURE_INIT();
     TL_REQUIRE(out && q && cache_k && cache_v, "%s: null pointer", name);
     TL_REQUIRE(T >= 1 && n_heads >= 1, "%s: bad sizes T=%d n_heads=%d", name, T, n_heads);
@@ -352,8 +410,9 @@ static int launch_decode_attention(void* out, const void* q, void* cache_k, void
     dim3 grid(n_heads, n_chunks);
     hipStream_t st = tl::stream();
     auto launch = [&](auto kernel) {
-        hipLaunchKernelGGL(kernel, grid, dim3(tl::kAttnThreads), 0, st, (tl::half_t*)out, ws, (const tl::half_t*)q,
-                           (tl::half_t*)cache_k, (tl::half_t*)cache_v, T, n_heads, inv_scale, n_chunks);
+        hipLaunchKernelGGL(kernel, grid, dim3(tl::kAttnThreads), 0, st, (tl::half_t*)out, ws,
+                           (const tl::half_t*)q, (tl::half_t*)cache_k, (tl::half_t*)cache_v,
+                           (const tl::half_t*)rope_table, T, n_heads, inv_scale, n_chunks);
     };
     if (fuse_rope) {
         if (head_dim == 64) launch(tl::decode_attn_partial_kernel<8, true>);
@@ -375,15 +434,27 @@ static int launch_decode_attention(void* out, const void* q, void* cache_k, void
 
 int tl_decode_attention_f16(void* out, const void* q, const void* cache_k, const void* cache_v, int T, int n_heads,
                             int head_dim) {
-    return launch_decode_attention(out, q, const_cast<void*>(cache_k), const_cast<void*>(cache_v), T, n_heads, head_dim,
-                                   false, "tl_decode_attention_f16");
+    return launch_decode_attention(out, q, const_cast<void*>(cache_k), const_cast<void*>(cache_v), nullptr, T, n_heads,
+                                   head_dim, false, "tl_decode_attention_f16");
 }
 
-int tl_decode_attention_rope_f16(void* out, const void* qkv, void* cache_k, void* cache_v, int pos, int n_heads,
-                                 int head_dim) {
+int tl_decode_attention_rope_f16(void* out, const void* qkv, void* cache_k, void* cache_v, const void* rope_table,
+                                 int pos, int n_heads, int head_dim) {
     TL_REQUIRE(pos >= 0, "tl_decode_attention_rope_f16: negative position");
-    return launch_decode_attention(out, qkv, cache_k, cache_v, pos + 1, n_heads, head_dim, true,
+    TL_REQUIRE(rope_table == nullptr || tl::aligned16(rope_table), "tl_decode_attention_rope_f16: misaligned table");
+    return launch_decode_attention(out, qkv, cache_k, cache_v, rope_table, pos + 1, n_heads, head_dim, true,
                                    "tl_decode_attention_rope_f16");
+}
+
+int tl_rope_table_f16(void* table, int max_seq, int head_dim) {
+    TL_ENSURE_INIT();
+    TL_REQUIRE(table, "tl_rope_table_f16: null pointer");
+    TL_REQUIRE(max_seq >= 1 && head_dim >= 2 && head_dim % 2 == 0, "tl_rope_table_f16: bad sizes");
+    const size_t n = (size_t)max_seq * (head_dim / 2);
+    hipLaunchKernelGGL(tl::rope_table_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, tl::stream(),
+                       (tl::half_t*)table, max_seq, head_dim);
+    TL_CHECK_LAUNCH("rope_table_kernel");
+    return TL_OK;
 }
 
 int tl_rope_qk_store_kv_f16(void* qkv, void* cache_k, void* cache_v, int pos, int n_heads, int head_dim) {

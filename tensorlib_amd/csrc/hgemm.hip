@@ -258,9 +258,6 @@ __global__ void __launch_bounds__(WM* WN * 64) hgemm_f16_dlds_kernel(HgemmArgs a
         b_src[j] = B + (size_t)gr * K + c * 8;
     }
     auto issue_loads = [&](int stage, int kt) {
-#if defined(TL_EXP_NOLOAD)
-        if (kt >= STAGES) return;
-#endif
         lds_byte_t* sa = lds + stage * STAGE_BYTES;
         lds_byte_t* sb = sa + A_BYTES;
         const size_t koff = (size_t)kt * BK;
@@ -328,10 +325,6 @@ __global__ void __launch_bounds__(WM* WN * 64) hgemm_f16_dlds_kernel(HgemmArgs a
             bf[j] = *reinterpret_cast<const half8_t*>(st + b_base + j * 32 * RB + fr_off[ks]);
     };
     auto mfmas = [&](const half8_t (&af)[MT], const half8_t (&bf)[NT]) {
-#if defined(TL_EXP_NOMFMA)
-        acc[0][0][0] += (float)af[0][0] + (float)bf[0][0];
-        return;
-#endif
 #pragma unroll
         for (int i = 0; i < MT; ++i)
 #pragma unroll
@@ -385,16 +378,12 @@ __global__ void __launch_bounds__(WM* WN * 64) hgemm_f16_dlds_kernel(HgemmArgs a
 #pragma unroll
             for (int e = 0; e < 16; ++e) {
                 const int row = m0 + wm * TM + i * 32 + 8 * (e / 4) + c_row_base + (e % 4);
-#if defined(TL_EXP_NOSTORE)
-                if (row < M && acc[i][j][e] == 123.456f) C[(size_t)row * N + col] = (half_t)acc[i][j][e];
-#else
                 if (row < M) {
                     if (a.partial)
                         a.partial[((size_t)blockIdx.z * M + row) * N + col] = acc[i][j][e];
                     else
                         C[(size_t)row * N + col] = (half_t)acc[i][j][e];
                 }
-#endif
             }
         }
     }

@@ -292,14 +292,21 @@ class HipDevice:
               "tl_decode_attention_f16")
         return out
 
-    def decode_attention_rope(self, qkv: torch.Tensor, cache_k: torch.Tensor, cache_v: torch.Tensor, pos: int):
+    def rope_table(self, max_seq: int, head_dim: int) -> torch.Tensor:
+        t = self.empty(max_seq, head_dim // 2, 2)
+        check(self.lib.tl_rope_table_f16(_ptr(t), max_seq, head_dim), "tl_rope_table_f16")
+        return t
+
+    def decode_attention_rope(self, qkv: torch.Tensor, cache_k: torch.Tensor, cache_v: torch.Tensor, pos: int,
+                              rope_table: torch.Tensor | None = None):
         """qkv: [3, n_heads, head_dim] raw projections of the token at `pos`; writes cache rows `pos`."""
         _req(qkv, name="qkv"), _req(cache_k, name="cache_k"), _req(cache_v, name="cache_v")
         _, H, D = qkv.shape
         if cache_k.shape[1:] != (H, D) or cache_v.shape != cache_k.shape or pos >= cache_k.shape[0]:
             raise ValueError("cache shape does not match qkv / pos")
         out = self.empty(H, D)
-        check(self.lib.tl_decode_attention_rope_f16(_ptr(out), _ptr(qkv), _ptr(cache_k), _ptr(cache_v), pos, H, D),
+        tab = ctypes.c_void_p(0) if rope_table is None else _ptr(_req(rope_table, name="rope_table"))
+        check(self.lib.tl_decode_attention_rope_f16(_ptr(out), _ptr(qkv), _ptr(cache_k), _ptr(cache_v), tab, pos, H, D),
               "tl_decode_attention_rope_f16")
         return out
 

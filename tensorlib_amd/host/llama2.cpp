@@ -75,6 +75,7 @@ struct tlm_model {
     std::vector<LayerWeights> layers;
     std::vector<Buf> cache_k, cache_v;  // per layer [max_seq, n_heads, head_dim]
     Buf x, x_norm, x_residual, qkv, x13, x2, scores, scores2, mask, xq_c, keys_c, values_c, s_v, o_c, logits;
+    Buf rope_table;  // [max_seq][head_dim/2][cos, sin], filled once at creation
     std::vector<void*> owned_weights;  // device allocations made by tlm_load_checkpoint
     int* d_tokens = nullptr;   // [max_tokens + generated]
     int d_tokens_cap = 0;
@@ -179,7 +180,8 @@ struct tlm_model {
                 gemv(x_norm.p, w.wv, xv(1), dim, dim);
             }
             // RoPE(q), RoPE(k) -> cache_k[pos], v -> cache_v[pos] and the attention itself, cache read in place
-            ck(tl_decode_attention_rope_f16(o_c.p, qkv.p, cache_k[l].p, cache_v[l].p, pos, H, D), "decode_attention_rope");
+            ck(tl_decode_attention_rope_f16(o_c.p, qkv.p, cache_k[l].p, cache_v[l].p, rope_table.p, pos, H, D),
+               "decode_attention_rope");
             gemv(o_c.p, w.wo, x_norm.p, dim, dim);
             // h = x + attn ; x_norm = rmsnorm(h) * ffn_norm
             ck(tl_add_rms_norm_f16(x_residual.p, x_norm.p, x.p, x_norm.p, w.ffn_norm, eps, dim, 1), "add_rms_norm");
@@ -265,6 +267,8 @@ int tlm_create(tlm_model** out, int dim, int hidden_dim, int n_layers, int n_hea
         m->keys_c.alloc((size_t)max_seq_len * dim);
         m->values_c.alloc((size_t)max_seq_len * dim);
         m->logits.alloc(S * vocab_size);
+        m->rope_table.alloc((size_t)max_seq_len * (dim / n_heads));
+        ck(tl_rope_table_f16(m->rope_table.p, max_seq_len, dim / n_heads), "rope_table");
         m->d_tokens_cap = max_seq_len + 8;
         void* p = nullptr;
         ck(tl_malloc(&p, (size_t)m->d_tokens_cap * sizeof(int)), "tl_malloc tokens");
@@ -282,7 +286,7 @@ int tlm_destroy(tlm_model* m) {
     for (auto& b : m->cache_k) b.release();
     for (auto& b : m->cache_v) b.release();
     for (Buf* b : {&m->x, &m->x_norm, &m->x_residual, &m->qkv, &m->x13, &m->x2, &m->scores, &m->scores2, &m->mask,
-                   &m->xq_c, &m->keys_c, &m->values_c, &m->s_v, &m->o_c, &m->logits})
+                   &m->xq_c, &m->keys_c, &m->values_c, &m->s_v, &m->o_c, &m->logits, &m->rope_table})
         b->release();
     if (m->d_tokens) tl_free(m->d_tokens);
     for (void* p : m->owned_weights) tl_free(p);

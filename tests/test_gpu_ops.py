@@ -243,6 +243,11 @@ def test_decode_attention_rope_equals_separate_steps(dev, oracle, pos, H, D):
     got = dev.decode_attention_rope(q2, k2, v2, pos).cpu().numpy()
     assert np.array_equal(got.view(np.uint16), want.view(np.uint16))
     assert torch.equal(k1, k2) and torch.equal(v1, v2)
+    # with the precomputed (cos, sin) table: same bits again
+    q3, k3, v3 = dev.from_numpy(qkv), dev.from_numpy(ck0), dev.from_numpy(cv0)
+    got3 = dev.decode_attention_rope(q3, k3, v3, pos, rope_table=dev.rope_table(S, D)).cpu().numpy()
+    assert np.array_equal(got3.view(np.uint16), want.view(np.uint16))
+    assert torch.equal(k1, k3) and torch.equal(v1, v3)
     assert np.array_equal(q2.cpu().numpy().view(np.uint16), qkv.view(np.uint16))   # raw projections untouched
     # and against the CPU chain
     q_rot = oracle.rope(qkv[0].reshape(1, 1, H, D), pos).reshape(H, D)
@@ -272,3 +277,25 @@ def test_gemv_silu_mul_limits(dev):
         dev.gemv_silu_mul(dev.empty(2 * 16384), dev.empty(8, 16384))     # K beyond the fused kernel's limit
     with pytest.raises(TensorLibError):
         dev.gemv_silu_mul(dev.empty(2 * 100), dev.empty(8, 100))         # K not a multiple of 8
+
+
+def test_rope_table_values(dev):
+    D, S = 128, 300
+    tab = dev.rope_table(S, D).cpu().numpy().astype(np.float64)
+    pos = np.arange(S)[:, None]
+    th = pos * 10000.0 ** (-2.0 * np.arange(D // 2)[None, :] / D)
+    assert np.abs(tab[..., 0] - np.cos(th)).max() < 1.5e-3 and np.abs(tab[..., 1] - np.sin(th)).max() < 1.5e-3
+    assert np.all(tab[0, :, 0] == 1.0) and np.all(tab[0, :, 1] == 0.0)
+
+
+def test_decode_attention_repeated_calls_reuse_counters(dev, oracle):
+    """The chunk-merge tickets must be back at zero after every launch: many calls in a row, with
+    different numbers of chunks, all have to agree with the CPU chain."""
+    H, D = 8, 128
+    q = synth.normal_f16(140, (H, D), 1.0)
+    ck = synth.normal_f16(141, (700, H, D), 1.0)
+    cv = synth.normal_f16(142, (700, H, D), 1.0)
+    qd, kd, vd = dev.from_numpy(q), dev.from_numpy(ck), dev.from_numpy(cv)
+    for T in (700, 65, 700, 130, 64, 129, 700):
+        got = dev.decode_attention(qd, kd, vd, T).cpu().numpy()
+        assert_close_f16(got, _attention_chain_oracle(oracle, q, ck, cv, T), RTOL, 2e-3, f"repeat T={T}")
