@@ -17,6 +17,7 @@
 // registers and are written to the other buffer before the single barrier of the step.
 #include <cstring>
 #include <mutex>
+#include <type_traits>
 
 #include "tl_internal.h"
 
@@ -191,6 +192,17 @@ __global__ void __launch_bounds__(WM* WN * 64) hgemm_f16_mfma_kernel(HgemmArgs a
 // rows fill one 256-byte LDS line and CPR is the number of chunks per row.  The 16 rows a
 // ds_read_b128 group touches then land in 16 different 16-byte bank groups.
 // Requirements: K % BK == 0 (no zero fill is possible on this path), K % 8 == 0, aligned operands.
+// One global_load_lds_dwordx4: lane l's 16 bytes at `src` go to LDS bytes [dst + 16*l, +16).
+// Written as inline assembly on purpose: the compiler models this instruction as a flat access that may
+// touch LDS, and while one is outstanding (always, in a ring whose vmcnt waits it cannot see) it turns
+// every wait for ds_read data into lgkmcnt(0), including reads issued an instant earlier.  Hidden from
+// it, the ds_reads are the only lgkmcnt traffic and get exact in-order counts.
+__device__ __forceinline__ void load_16B_per_lane_to_lds(const half_t* src,
+                                                         __attribute__((address_space(3))) unsigned char* dst) {
+    const unsigned lds_addr = (unsigned)(unsigned long)dst;
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(src), "s"(lds_addr) : "memory");
+}
+
 template <int N_>
 __device__ __forceinline__ void wait_vmcnt_and_barrier() {
     // waits until at most N_ of this wavefront's global->LDS loads are outstanding and all of its
@@ -199,7 +211,9 @@ __device__ __forceinline__ void wait_vmcnt_and_barrier() {
     asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(N_) : "memory");
 }
 
-template <int BM, int BN, int BK, int WM, int WN, int STAGES, bool PIPE>
+// MODE 0: every wavefront reads the fragments of a K step, then issues its MFMAs.
+// MODE 1: fragments double buffered in registers across K steps.
+template <int BM, int BN, int BK, int WM, int WN, int STAGES, int MODE>
 __global__ void __launch_bounds__(WM* WN * 64) hgemm_f16_dlds_kernel(HgemmArgs a) {
     constexpr int NW = WM * WN;
     constexpr int RB = BK * 2;                 // bytes per tile row
@@ -216,7 +230,7 @@ __global__ void __launch_bounds__(WM* WN * 64) hgemm_f16_dlds_kernel(HgemmArgs a
     constexpr int KS = BK / 16;
     static_assert(BK == 32 || BK == 64, "BK must be 32 or 64");
     static_assert(BM % (RPW * NW) == 0 && BN % (RPW * NW) == 0, "tile rows must split over the wavefronts");
-    static_assert(STAGES >= 2 && STAGES <= 4 && LPW * (STAGES - 2) < 64, "vmcnt is a 6-bit counter");
+    static_assert(STAGES >= 2 && STAGES <= 5 && LPW * (STAGES - 2) < 64, "vmcnt is a 6-bit counter");
 
     extern __shared__ __attribute__((aligned(1024))) unsigned char smem_raw[];
     typedef __attribute__((address_space(3))) unsigned char lds_byte_t;
@@ -235,6 +249,11 @@ __global__ void __launch_bounds__(WM* WN * 64) hgemm_f16_dlds_kernel(HgemmArgs a
     const half_t* __restrict__ B = a.B + (size_t)batch * a.sb;
     half_t* __restrict__ C = a.C + (size_t)batch * a.sc;
     const int M = a.M, N = a.N, K = a.K;
+    // Every kernel argument is pulled into registers here.  A scalar load still pending inside the main
+    // loop would make the compiler treat lgkmcnt as unordered and turn every wait for LDS data into
+    // lgkmcnt(0), which also waits for the fragment reads issued just before it.
+    float* const partial = a.partial;
+    asm volatile("" ::"s"(partial), "s"(C), "s"(M), "s"(N), "s"(a.kt_per_split));
 
     // ---- loader: wavefront-load j of this wavefront covers tile rows (j*NW + wave)*RPW .. +RPW ----
     const int ld_row_in_group = lane / CPR;
@@ -257,20 +276,21 @@ __global__ void __launch_bounds__(WM* WN * 64) hgemm_f16_dlds_kernel(HgemmArgs a
         gr = gr < N ? gr : N - 1;
         b_src[j] = B + (size_t)gr * K + c * 8;
     }
-    auto issue_loads = [&](int stage, int kt) {
-        lds_byte_t* sa = lds + stage * STAGE_BYTES;
-        lds_byte_t* sb = sa + A_BYTES;
+    auto a_off = [&](int kt) { return (kt % STAGES) * STAGE_BYTES; };
+    auto b_off = [&](int kt) { return (kt % STAGES) * STAGE_BYTES + A_BYTES; };
+    auto issue_a = [&](int kt) {
+        lds_byte_t* sa = lds + a_off(kt);
         const size_t koff = (size_t)kt * BK;
 #pragma unroll
         for (int j = 0; j < A_LOADS; ++j)
-            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(a_src[j] + koff),
-                                             (__attribute__((address_space(3))) void*)(sa + (j * NW + wave) * 1024), 16,
-                                             0, 0);
+            load_16B_per_lane_to_lds(a_src[j] + koff, sa + (j * NW + wave) * 1024);
+    };
+    auto issue_b = [&](int kt) {
+        lds_byte_t* sb = lds + b_off(kt);
+        const size_t koff = (size_t)kt * BK;
 #pragma unroll
         for (int j = 0; j < B_LOADS; ++j)
-            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(b_src[j] + koff),
-                                             (__attribute__((address_space(3))) void*)(sb + (j * NW + wave) * 1024), 16,
-                                             0, 0);
+            load_16B_per_lane_to_lds(b_src[j] + koff, sb + (j * NW + wave) * 1024);
     };
 
     // ---- fragment reader: row (lane % 32) of a 32-row MFMA tile, chunk 2*ks + lane/32 ----
@@ -280,7 +300,7 @@ __global__ void __launch_bounds__(WM* WN * 64) hgemm_f16_dlds_kernel(HgemmArgs a
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) fr_off[ks] = fr_row * RB + (((ks * 2 + (lane >> 5)) ^ fr_sw) * 16);
     const int a_base = wm * TM * RB;
-    const int b_base = A_BYTES + wn * TN * RB;
+    const int b_base = wn * TN * RB;
 
     float16_t acc[MT][NT];
 #pragma unroll
@@ -299,65 +319,75 @@ __global__ void __launch_bounds__(WM* WN * 64) hgemm_f16_dlds_kernel(HgemmArgs a
     for (int j = 0; j < B_LOADS; ++j) b_src[j] += (size_t)kt_begin * BK;
 #pragma unroll
     for (int s = 0; s < STAGES - 1; ++s)
-        if (s < KT) issue_loads(s, s);
+        if (s < KT) { issue_a(s); issue_b(s); }
 
     // Wait until tile kt has landed in LDS for every wavefront.  Tiles requested after kt
     // (at most STAGES-2 of them) may stay in flight.
     auto sync_for = [&](int kt) {
         const int ahead = (KT - 1 - kt) < (STAGES - 2) ? (KT - 1 - kt) : (STAGES - 2);
-        if constexpr (STAGES == 2) {
-            wait_vmcnt_and_barrier<0>();
-        } else if constexpr (STAGES == 3) {
-            if (ahead >= 1) wait_vmcnt_and_barrier<LPW>(); else wait_vmcnt_and_barrier<0>();
-        } else {
-            if (ahead >= 2) wait_vmcnt_and_barrier<2 * LPW>();
-            else if (ahead == 1) wait_vmcnt_and_barrier<LPW>();
-            else wait_vmcnt_and_barrier<0>();
-        }
+        if (STAGES >= 5 && ahead >= 3) wait_vmcnt_and_barrier<3 * LPW>();
+        else if (STAGES >= 4 && ahead == 2) wait_vmcnt_and_barrier<2 * LPW>();
+        else if (STAGES >= 3 && ahead == 1) wait_vmcnt_and_barrier<LPW>();
+        else wait_vmcnt_and_barrier<0>();
+    };
+    // After the barrier of tile kt every wavefront is done with tile kt-1: refill what it occupied.
+    auto issue_after_sync = [&](int kt) {
+        if (kt + STAGES - 1 < KT) { issue_a(kt + STAGES - 1); issue_b(kt + STAGES - 1); }
     };
     auto load_frags = [&](half8_t (&af)[MT], half8_t (&bf)[NT], int kt, int ks) {
-        const unsigned char* st = smem_raw + (kt % STAGES) * STAGE_BYTES;
+        const unsigned char* sa = smem_raw + a_off(kt) + a_base;
+        const unsigned char* sb = smem_raw + b_off(kt) + b_base;
 #pragma unroll
         for (int i = 0; i < MT; ++i)
-            af[i] = *reinterpret_cast<const half8_t*>(st + a_base + i * 32 * RB + fr_off[ks]);
+            af[i] = *reinterpret_cast<const half8_t*>(sa + i * 32 * RB + fr_off[ks]);
 #pragma unroll
         for (int j = 0; j < NT; ++j)
-            bf[j] = *reinterpret_cast<const half8_t*>(st + b_base + j * 32 * RB + fr_off[ks]);
+            bf[j] = *reinterpret_cast<const half8_t*>(sb + j * 32 * RB + fr_off[ks]);
     };
     auto mfmas = [&](const half8_t (&af)[MT], const half8_t (&bf)[NT]) {
 #pragma unroll
         for (int i = 0; i < MT; ++i)
 #pragma unroll
             for (int j = 0; j < NT; ++j)
-                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[i], bf[j], acc[i][j], 0, 0, 0);
+                // B's fragment goes in as the first operand: the accumulator then holds the tile
+                // transposed, i.e. lane l owns row (l % 32) of C and, per group of four accumulator
+                // registers, four CONSECUTIVE columns, which is what a vector store wants.
+                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(bf[j], af[i], acc[i][j], 0, 0, 0);
     };
 
-    if constexpr (PIPE) {
+    if constexpr (MODE == 1) {
         // Fragments are double buffered in registers: the ds_reads of K step s+1 (or of the
         // next tile's first step, after the tile barrier) are issued before the MFMAs of step s.
         static_assert(KS % 2 == 0, "fragment ping-pong needs an even number of K steps");
         half8_t af[2][MT], bf[2][NT];
         sync_for(0);
-        if (STAGES - 1 < KT) issue_loads((STAGES - 1) % STAGES, STAGES - 1);
+        issue_after_sync(0);
         load_frags(af[0], bf[0], 0, 0);
-        for (int kt = 0; kt < KT; ++kt) {
+        // The last tile is peeled off so that inside the loop the fragments of the next tile are always
+        // requested: the compiler then knows how many reads are younger than the ones an MFMA needs.
+        auto tile = [&](int kt, auto has_next) {
 #pragma unroll
             for (int ks = 0; ks < KS; ++ks) {
                 const int cur = ks & 1, nxt = cur ^ 1;
                 if (ks + 1 < KS) {
                     load_frags(af[nxt], bf[nxt], kt, ks + 1);
-                } else if (kt + 1 < KT) {
+                } else if constexpr (decltype(has_next)::value) {
                     sync_for(kt + 1);  // every wavefront holds its last fragments of tile kt in registers
-                    if (kt + STAGES < KT) issue_loads((kt + STAGES) % STAGES, kt + STAGES);
+                    issue_after_sync(kt + 1);
                     load_frags(af[nxt], bf[nxt], kt + 1, 0);
                 }
+                // keep the reads of the next step ahead of this step's MFMAs, so they land under them
+                __builtin_amdgcn_sched_barrier(0);
                 mfmas(af[cur], bf[cur]);
+                __builtin_amdgcn_sched_barrier(0);
             }
-        }
+        };
+        for (int kt = 0; kt + 1 < KT; ++kt) tile(kt, std::true_type{});
+        if (KT > 0) tile(KT - 1, std::false_type{});
     } else {
         for (int kt = 0; kt < KT; ++kt) {
             sync_for(kt);
-            if (kt + STAGES - 1 < KT) issue_loads((kt + STAGES - 1) % STAGES, kt + STAGES - 1);
+            issue_after_sync(kt);
 #pragma unroll
             for (int ks = 0; ks < KS; ++ks) {
                 half8_t af[MT], bf[NT];
@@ -367,25 +397,78 @@ __global__ void __launch_bounds__(WM* WN * 64) hgemm_f16_dlds_kernel(HgemmArgs a
         }
     }
 
-    const int c_col = lane & 31;
-    const int c_row_base = (lane >> 5) * 4;
+    // ---- epilogue.  acc[i][j][4*g + r] = C[row i*32 + lane%32][col j*32 + 8*g + 4*(lane/32) + r] ----
+    const int e_row = lane & 31;
+    const int e_col = (lane >> 5) * 4;
+    const int row_base = m0 + wm * TM, col_base = n0 + wn * TN;
+    if (partial) {
+        // split-K: fp32 partial sums, four consecutive columns (16 bytes) per store where the row allows it
+        const bool vec = (N % 4) == 0;
 #pragma unroll
-    for (int i = 0; i < MT; ++i) {
+        for (int i = 0; i < MT; ++i) {
+            const int row = row_base + i * 32 + e_row;
+            if (row >= M) continue;
+            float* prow = partial + ((size_t)blockIdx.z * M + row) * N;
 #pragma unroll
-        for (int j = 0; j < NT; ++j) {
-            const int col = n0 + wn * TN + j * 32 + c_col;
-            if (col >= N) continue;
+            for (int j = 0; j < NT; ++j)
 #pragma unroll
-            for (int e = 0; e < 16; ++e) {
-                const int row = m0 + wm * TM + i * 32 + 8 * (e / 4) + c_row_base + (e % 4);
-                if (row < M) {
-                    if (a.partial)
-                        a.partial[((size_t)blockIdx.z * M + row) * N + col] = acc[i][j][e];
-                    else
-                        C[(size_t)row * N + col] = (half_t)acc[i][j][e];
+                for (int g = 0; g < 4; ++g) {
+                    const int col = col_base + j * 32 + g * 8 + e_col;
+                    if (vec && col + 3 < N) {
+                        float4_t v = {acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]};
+                        *reinterpret_cast<float4_t*>(prow + col) = v;
+                    } else {
+#pragma unroll
+                        for (int r = 0; r < 4; ++r)
+                            if (col + r < N) prow[col + r] = acc[i][j][4 * g + r];
+                    }
                 }
+        }
+        return;
+    }
+    if ((N % 8) == 0 && (reinterpret_cast<uintptr_t>(C) & 15u) == 0) {
+        // fp16 output through LDS: every wavefront turns 32 x TN blocks of its accumulators into row-major
+        // halves in a private LDS region (8-byte writes), reads them back 16 bytes per lane and stores
+        // whole 16-byte pieces of C rows (TN = 64: full 128-byte lines).  Rows are padded by 16 bytes so
+        // that the 32 rows of one write land in different banks.
+        constexpr int RS = TN * 2 + 16;          // bytes per staged row
+        constexpr int CH = TN / 8;               // 16-byte chunks per row
+        constexpr int RPR = 64 / CH;             // rows per wavefront-wide read
+        static_assert(NW * 32 * RS <= STAGES * STAGE_BYTES, "staging area must fit the ring");
+        // all wavefronts are done with the operand tiles before anyone overwrites them
+        asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+        unsigned char* region = smem_raw + wave * (32 * RS);
+#pragma unroll
+        for (int i = 0; i < MT; ++i) {
+#pragma unroll
+            for (int j = 0; j < NT; ++j)
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    half4_t h = {(half_t)acc[i][j][4 * g], (half_t)acc[i][j][4 * g + 1], (half_t)acc[i][j][4 * g + 2],
+                                 (half_t)acc[i][j][4 * g + 3]};
+                    *reinterpret_cast<half4_t*>(region + e_row * RS + (j * 32 + g * 8 + e_col) * 2) = h;
+                }
+#pragma unroll
+            for (int q = 0; q < 32 / RPR; ++q) {
+                const int r = q * RPR + lane / CH, c = lane % CH;
+                const half8_t v = *reinterpret_cast<const half8_t*>(region + r * RS + c * 16);
+                const int row = row_base + i * 32 + r, col = col_base + c * 8;
+                if (row < M && col < N) *reinterpret_cast<half8_t*>(C + (size_t)row * N + col) = v;
             }
         }
+        return;
+    }
+#pragma unroll
+    for (int i = 0; i < MT; ++i) {
+        const int row = row_base + i * 32 + e_row;
+        if (row >= M) continue;
+#pragma unroll
+        for (int j = 0; j < NT; ++j)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                const int col = col_base + j * 32 + (e / 4) * 8 + e_col + (e % 4);
+                if (col < N) C[(size_t)row * N + col] = (half_t)acc[i][j][e];
+            }
     }
 }
 
@@ -451,10 +534,10 @@ struct HgemmVariant {
     { "t" #BM "x" #BN "x" #BK "w" #WM "x" #WN, BM, BN, BK, WM * WN * 64, 0, hgemm_f16_mfma_kernel<BM, BN, BK, WM, WN> }
 #define TL_HGEMM_DLDS(BM, BN, BK, WM, WN, ST) \
     { "d" #BM "x" #BN "x" #BK "w" #WM "x" #WN "s" #ST, BM, BN, BK, WM * WN * 64, ST, \
-      hgemm_f16_dlds_kernel<BM, BN, BK, WM, WN, ST, false> }
+      hgemm_f16_dlds_kernel<BM, BN, BK, WM, WN, ST, 0> }
 #define TL_HGEMM_PIPE(BM, BN, BK, WM, WN, ST) \
     { "p" #BM "x" #BN "x" #BK "w" #WM "x" #WN "s" #ST, BM, BN, BK, WM * WN * 64, ST, \
-      hgemm_f16_dlds_kernel<BM, BN, BK, WM, WN, ST, true> }
+      hgemm_f16_dlds_kernel<BM, BN, BK, WM, WN, ST, 1> }
 
 static const HgemmVariant g_variants[] = {
     {"auto", 0, 0, 0, 0, 0, nullptr},
@@ -540,11 +623,12 @@ static int hgemm_variant_index(const char* name) {
 }
 
 // Measured on MI355X over the Llama2-7B prefill shapes (M in {128,512,2048}):
-//   >= ~0.9 x CUs tiles of 256x256 : 256x256x64, 8 wavefronts (128x64 each), 2-stage LDS ring
+//   >= ~0.9 x CUs tiles of 256x256 : 256x256x64, 8 wavefronts (128x64 each), 2-stage LDS ring, fragments
+//                                    double buffered
 //   M >= 1024 otherwise            : 128x256x64, 8 wavefronts, fragments double buffered
 //   fewer rows                     : 128x128x64, 8 wavefronts, plus split-K (see launch_hgemm)
 static int pick_variant(size_t M, size_t N, size_t K, int cus) {
-    static const int v_big = hgemm_variant_index("d256x256x64w2x4s2");
+    static const int v_big = hgemm_variant_index("p256x256x64w2x4s2");
     static const int v_mid = hgemm_variant_index("p128x256x64w2x4s2");
     static const int v_small = hgemm_variant_index("p128x128x64w2x4s2");
     (void)K;
