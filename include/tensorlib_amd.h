@@ -186,6 +186,15 @@ int tl_decode_attention_f16(void* out, const void* q, const void* cache_k, const
  * fp16 once, as tl_silu_mul_f16 would store it.  Needs 512 <= K <= 12288, K % 8 == 0. */
 int tl_gemv_silu_mul_f16(const void* ab, const void* W, void* y, size_t N, size_t K);
 
+/* y[N] = W[N,K] . (rmsnorm(x + addend) * norm_weight) and sum_out = x + addend: the residual EwiseAdd of
+ * TransformerBlock::forward, the RMSNorm that follows it and the Linear that consumes the norm
+ * (model/llama2_7b/src/Transformer.cpp:165-175, tensorLib/src/nn/rmsNorm.cpp:85-106) in one launch.
+ * The sum is rounded to fp16 before it is squared and the normalised vector is rounded to fp16 once, as
+ * tl_add_rms_norm_f16 stores them.  addend may be NULL (plain RMSNorm), sum_out may be NULL; sum_out must
+ * not alias x or addend.  Needs 512 <= K <= 12288, K % 8 == 0, 16-byte aligned operands. */
+int tl_gemv_add_rms_norm_f16(const void* x, const void* addend, const void* norm_weight, float eps,
+                             const void* W, void* y, void* sum_out, size_t N, size_t K);
+
 /* tl_rope_qk_store_kv_f16 + tl_decode_attention_f16 in one launch pair: qkv is the raw q|k|v
  * projection of the token at position `pos`; q is rotated on load, the rotated k and the v row
  * are written to cache_k[pos] / cache_v[pos], and out[h,:] attends to positions 0..pos.

@@ -89,6 +89,11 @@ struct GemvArgs {
     int K8;             // 16-byte chunks per row (K / 8)
     int num_row_blocks; // ceil(N / rows per workgroup pass)
     long sx8, sw8, sy;  // batch strides: x and W in 16-byte chunks, y in elements
+    // XMODE 3 only: the vector that is multiplied is rmsnorm(x + x2) * g
+    const half8_t* x2;  // may be null (no addend)
+    const half8_t* g;   // norm weight
+    half8_t* sum_out;   // may be null; receives half(x + x2), written by workgroup 0
+    float eps;
 };
 
 // One wavefront per row group.  Dynamic LDS: K8 chunks of x (+ partial sums when KSPLIT > 1).
@@ -192,7 +197,12 @@ __global__ void __launch_bounds__(WAVES * 64) gemv_f16_wave_kernel(GemvArgs a) {
 //            the first W tile is requested before the staging barrier.
 //   XMODE 1: every wavefront reads its own K segment of x straight into registers.
 //   XMODE 2: like 1, but x is silu(a) * b of a [a | b] input (the SwiGLU gate fused into the load).
-// Dynamic LDS: [K8 chunks of x when XMODE == 0] + 2*RG*KSPLIT*ROWS floats when KSPLIT > 1.
+//   XMODE 3: like 1, but x is rmsnorm(h + d) * g: every wavefront forms half(h + d) of its K segment,
+//            the KSPLIT segment sums of squares meet in LDS (fixed order), and the normalised, weighted
+//            vector is rounded to fp16 once, as the separate add + RMSNorm kernel would have stored it.
+//            Workgroup 0 also writes half(h + d) out (the new residual stream).
+// Dynamic LDS: [K8 chunks of x when XMODE == 0] + 2*RG*KSPLIT*ROWS floats when KSPLIT > 1
+//              (+ WAVES floats when XMODE == 3).
 template <int WAVES, int ROWS, int UNROLL, int KSPLIT, int XMODE>
 __global__ void __launch_bounds__(WAVES * 64) gemv_f16_stream_kernel(GemvArgs a) {
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
@@ -245,6 +255,24 @@ __global__ void __launch_bounds__(WAVES * 64) gemv_f16_stream_kernel(GemvArgs a)
         }
     }
 
+    half8_t gv[XMODE == 3 ? UNROLL : 1];
+    float ss = 0.f;
+    if constexpr (XMODE == 3) {
+        const half8_t* __restrict__ x2 = a.x2;
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u) {
+            const half8_t va = ok[u] ? x[cidx[u]] : zero8;
+            const half8_t vb = (ok[u] && x2) ? x2[cidx[u]] : zero8;
+            gv[u] = ok[u] ? a.g[cidx[u]] : zero8;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const half_t h = (half_t)((float)va[i] + (float)vb[i]);
+                xv[u][i] = h;
+                ss = __builtin_fmaf((float)h, (float)h, ss);
+            }
+        }
+    }
+
     half8_t cur[ROWS][UNROLL], nxt[ROWS][UNROLL];
     auto load_tile = [&](half8_t (&t)[ROWS][UNROLL], int rb) {
         const int row0 = (rb * RG + rgrp) * ROWS;
@@ -266,6 +294,24 @@ __global__ void __launch_bounds__(WAVES * 64) gemv_f16_stream_kernel(GemvArgs a)
         __syncthreads();
 #pragma unroll
         for (int u = 0; u < UNROLL; ++u) xv[u] = xs[ok[u] ? cidx[u] : 0];
+    }
+    if constexpr (XMODE == 3) {
+        // the first W tile is already in flight; finish the norm under its latency
+        float* nrm = part + (KSPLIT > 1 ? 2 * RG * KSPLIT * ROWS : 0);
+        ss = wave_sum(ss);
+        if (lane == 0) nrm[wave] = ss;
+        __syncthreads();
+        float total = 0.f;
+#pragma unroll
+        for (int sgm = 0; sgm < KSPLIT; ++sgm) total += nrm[rgrp * KSPLIT + sgm];
+        const float rs = 1.0f / sqrtf(total / (float)(K8 * 8) + a.eps);
+        const bool writer = blockIdx.x == 0 && rgrp == 0 && a.sum_out != nullptr;
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u) {
+            if (writer && ok[u]) a.sum_out[cidx[u]] = xv[u];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) xv[u][i] = (half_t)((float)xv[u][i] * rs * (float)gv[u][i]);
+        }
     }
 
     int it = 0;
@@ -409,6 +455,8 @@ static const GemvVariant g_variants[] = {
     TL_STREAM2(4, 1, 2, 4),       // 49, 50
     TL_STREAM(4, 2, 2, 4, 2),     // 51  silu*mul prologue, K <= 4096
     TL_STREAM(8, 2, 3, 8, 2),     // 52  silu*mul prologue, K <= 12288
+    TL_STREAM(4, 2, 2, 4, 3),     // 53  add + RMSNorm prologue, K <= 4096
+    TL_STREAM(8, 2, 3, 8, 3),     // 54  add + RMSNorm prologue, K <= 12288
 };
 static constexpr int kNumVariants = sizeof(g_variants) / sizeof(g_variants[0]);
 static int g_forced_variant = 0;
@@ -442,7 +490,7 @@ static int pick_variant(size_t N, size_t K, int* waves_per_cu) {
 }
 
 int launch_gemv(const void* x, const void* W, void* y, size_t N, size_t K, size_t batch, size_t sx,
-                size_t sw, size_t sy, int prologue) {
+                size_t sw, size_t sy, int prologue, const GemvNormPrologue* norm) {
     if (N == 0 || batch == 0) return TL_OK;
     TL_REQUIRE(N <= 0x7fffffffu && K <= 0x7fffffffu && batch <= 65535, "gemv: size out of range");
     const DeviceInfo& dev = device_info();
@@ -475,6 +523,10 @@ int launch_gemv(const void* x, const void* W, void* y, size_t N, size_t K, size_
     a.sx8 = (long)(sx / 8);
     a.sw8 = (long)(sw / 8);
     a.sy = (long)sy;
+    a.x2 = norm ? (const half8_t*)norm->addend : nullptr;
+    a.g = norm ? (const half8_t*)norm->weight : nullptr;
+    a.sum_out = norm ? (half8_t*)norm->sum_out : nullptr;
+    a.eps = norm ? norm->eps : 0.f;
 
     if (a.K8 < 64 && g_forced_variant == 0) {
         int lpr = a.K8 >= 32 ? 32 : a.K8 >= 16 ? 16 : 8;
@@ -503,6 +555,17 @@ int launch_gemv(const void* x, const void* W, void* y, size_t N, size_t K, size_
         else if (a.K8 <= 1536) { vi = v_k12288; auto_wpc = 16; }
         else return set_error(TL_ELIMIT, "gemv with fused silu*mul: K=%zu exceeds 12288", K);
     }
+    if (prologue == 2) {
+        static const int v_k4096 = variant_index("stream_w4r2u2s4x3");
+        static const int v_k12288 = variant_index("stream_w8r2u3s8x3");
+        TL_REQUIRE(norm && norm->weight && batch == 1, "gemv with fused add + RMSNorm: needs a norm weight, batch 1");
+        // every workgroup repeats the prologue (3 vectors from L2), so the grid is capped and loops
+        if (a.K8 <= 512) { vi = v_k4096; auto_wpc = 32; }
+        else if (a.K8 <= 1536) { vi = v_k12288; auto_wpc = 16; }
+        else return set_error(TL_ELIMIT, "gemv with fused add + RMSNorm: K=%zu exceeds 12288", K);
+    }
+    TL_REQUIRE(g_variants[vi].xmode != 3 || prologue == 2,
+               "gemv variant %s cannot hold a plain x: it needs the add + RMSNorm operands", g_variants[vi].name);
     TL_REQUIRE(g_variants[vi].xmode != 2 || prologue == 1,
                "gemv variant %s cannot hold a plain x: it reads an [a | b] input of 2*K halves", g_variants[vi].name);
     if (g_variants[vi].xmode >= 0) {
@@ -520,7 +583,8 @@ int launch_gemv(const void* x, const void* W, void* y, size_t N, size_t K, size_
     const int rows_per_block = rg * v.rows;
     a.num_row_blocks = (int)((N + rows_per_block - 1) / rows_per_block);
     size_t lds = (v.xmode >= 1 ? 0 : (size_t)a.K8 * 16) +
-                 (v.ksplit > 1 ? (size_t)(v.xmode >= 0 ? 2 : 1) * rg * v.ksplit * v.rows * 4 : 0);
+                 (v.ksplit > 1 ? (size_t)(v.xmode >= 0 ? 2 : 1) * rg * v.ksplit * v.rows * 4 : 0) +
+                 (v.xmode == 3 ? (size_t)v.waves * 4 : 0);
     if (lds > 64 * 1024) {
         // x does not fit the default LDS window: fall back to the generic kernel.
         int blocks = (int)((N + 3) / 4);
@@ -578,4 +642,17 @@ extern "C" int tl_gemv_silu_mul_f16(const void* ab, const void* W, void* y, size
                "tl_gemv_silu_mul_f16: needs K %% 8 == 0 and 16-byte aligned operands");
     TL_REQUIRE(K / 8 >= 64, "tl_gemv_silu_mul_f16: K=%zu too short for the fused kernel (K >= 512)", K);
     return tl::launch_gemv(ab, W, y, N, K, 1, 0, 0, 0, 1);
+}
+
+extern "C" int tl_gemv_add_rms_norm_f16(const void* x, const void* addend, const void* norm_weight, float eps,
+                                        const void* W, void* y, void* sum_out, size_t N, size_t K) {
+    TL_ENSURE_INIT();
+    TL_REQUIRE(x && norm_weight && W && y, "tl_gemv_add_rms_norm_f16: null pointer");
+    TL_REQUIRE(K % 8 == 0 && tl::aligned16(x) && tl::aligned16(W) && tl::aligned16(norm_weight) &&
+                   (!addend || tl::aligned16(addend)) && (!sum_out || tl::aligned16(sum_out)),
+               "tl_gemv_add_rms_norm_f16: needs K %% 8 == 0 and 16-byte aligned operands");
+    TL_REQUIRE(K / 8 >= 64, "tl_gemv_add_rms_norm_f16: K=%zu too short for the fused kernel (K >= 512)", K);
+    TL_REQUIRE(!sum_out || (sum_out != x && sum_out != addend), "tl_gemv_add_rms_norm_f16: sum_out must not alias an input");
+    tl::GemvNormPrologue np{addend, norm_weight, sum_out, eps};
+    return tl::launch_gemv(x, W, y, N, K, 1, 0, 0, 0, 2, &np);
 }

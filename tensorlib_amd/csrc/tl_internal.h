@@ -41,8 +41,16 @@ int ensure_init();
 int launch_fill_f16(void* out, uint16_t bits, size_t n);
 
 // Shared launchers (batch strides in elements; batch == 1 ignores them).
+// prologue 0: plain x; 1: x is [a | b], the multiplied vector is silu(a) * b; 2: the multiplied vector is
+// rmsnorm(x + norm->addend) * norm->weight and norm->sum_out receives half(x + addend).
+struct GemvNormPrologue {
+    const void* addend;  // may be null
+    const void* weight;
+    void* sum_out;       // may be null
+    float eps;
+};
 int launch_gemv(const void* x, const void* W, void* y, size_t N, size_t K, size_t batch, size_t sx,
-                size_t sw, size_t sy, int prologue);
+                size_t sw, size_t sy, int prologue, const GemvNormPrologue* norm = nullptr);
 int launch_hgemm(const void* A, const void* B, void* C, size_t M, size_t N, size_t K, size_t batch,
                  size_t sa, size_t sb, size_t sc);
 

@@ -336,6 +336,22 @@ class HipDevice:
         check(self.lib.tl_gemv_silu_mul_f16(_ptr(ab), _ptr(W), _ptr(y), N, K), "tl_gemv_silu_mul_f16")
         return y
 
+    def gemv_add_rms_norm(self, x: torch.Tensor, addend, weight: torch.Tensor, eps: float, W: torch.Tensor,
+                          want_sum: bool = True):
+        """(y, x + addend) with y = W . (rmsnorm(x + addend) * weight); addend may be None."""
+        _req(x, name="x"), _req(weight, name="weight"), _req(W, name="W")
+        if addend is not None:
+            _req(addend, name="addend")
+        N, K = W.shape
+        if x.numel() != K or weight.numel() != K or (addend is not None and addend.numel() != K):
+            raise ValueError("x, addend and weight must hold K elements")
+        y = self.empty(N)
+        s = self.empty(K) if want_sum else None
+        check(self.lib.tl_gemv_add_rms_norm_f16(_ptr(x), _ptr(addend) if addend is not None else None, _ptr(weight),
+                                                float(eps), _ptr(W), _ptr(y), _ptr(s) if s is not None else None, N, K),
+              "tl_gemv_add_rms_norm_f16")
+        return y, s
+
     # -- tuning hooks -------------------------------------------------------------------
     def set_gemv_variant(self, v: int) -> None:
         check(self.lib.tl_set_gemv_variant(v), "tl_set_gemv_variant")

@@ -17,6 +17,7 @@
 #include <memory>
 #include <stdexcept>
 #include <string>
+#include <utility>
 #include <vector>
 
 #include "tensorlib_amd.h"
@@ -166,7 +167,63 @@ struct tlm_model {
     // ---- fused single-token step --------------------------------------------------------------
     void gemv(const half* xin, const half* W, half* y, size_t N, size_t K) { ck(tl_gemv_f16(xin, W, y, N, K), "gemv"); }
 
+    // One decode step with the residual add and the RMSNorm folded into the operand load of the GEMV that
+    // consumes them: per layer qkv GEMV -> attention -> wo GEMV -> w1|w3 GEMV -> w2 GEMV.  Returns with the
+    // logits computed; the final hidden state ends in x.
     void decode_fused(int pos) {
+        const int H = n_heads, D = head_dim;
+        const bool norm_in_gemv = dim % 8 == 0 && dim >= 512 && dim <= 12288;
+        if (!norm_in_gemv) { decode_fused_separate_norm(pos); return; }
+        half* h = x.p;               // residual stream (current)
+        half* h_other = x_residual.p;
+        const half* delta = nullptr; // what still has to be added to h
+        half* attn_out = x_norm.p;   // wo's output
+        half* ffn_out = x2.p;        // w2's output (x2 is free: silu*mul happens inside w2's GEMV)
+        const bool ffn_fused = hidden % 8 == 0 && hidden >= 512 && hidden <= 12288;
+        if (!ffn_fused) ffn_out = o_c.p;  // x2 holds silu*mul then; o_c is free after wo
+        auto normed = [&](const half* norm_w, const half* W, half* y, size_t N, bool last_of_group) {
+            // every GEMV of a group (q, k, v or w1, w3) sees the same h and delta; the last one publishes the sum
+            half* sum_out = (delta && last_of_group) ? h_other : nullptr;
+            ck(tl_gemv_add_rms_norm_f16(h, delta, norm_w, eps, W, y, sum_out, N, dim), "gemv_add_rms_norm");
+            if (sum_out) { std::swap(h, h_other); delta = nullptr; }
+        };
+        for (int l = 0; l < n_layers; ++l) {
+            const LayerWeights& w = layers[l];
+            const size_t dd = (size_t)dim * dim;
+            if (w.wk == w.wq + dd && w.wv == w.wk + dd) {
+                normed(w.att_norm, w.wq, qkv.p, (size_t)3 * dim, true);
+            } else {
+                normed(w.att_norm, w.wq, xq(1), dim, false);
+                normed(w.att_norm, w.wk, xk(1), dim, false);
+                normed(w.att_norm, w.wv, xv(1), dim, true);
+            }
+            ck(tl_decode_attention_rope_f16(o_c.p, qkv.p, cache_k[l].p, cache_v[l].p, rope_table.p, pos, H, D),
+               "decode_attention_rope");
+            gemv(o_c.p, w.wo, attn_out, dim, dim);
+            delta = attn_out;
+            if (w.w3 == w.w1 + (size_t)hidden * dim) {
+                normed(w.ffn_norm, w.w1, x13.p, (size_t)2 * hidden, true);
+            } else {
+                normed(w.ffn_norm, w.w1, x1(1), hidden, false);
+                normed(w.ffn_norm, w.w3, x3(1), hidden, true);
+            }
+            if (ffn_fused) {
+                ck(tl_gemv_silu_mul_f16(x13.p, w.w2, ffn_out, dim, hidden), "gemv_silu_mul");
+            } else {
+                ck(tl_silu_mul_f16(x2.p, x1(1), x3(1), hidden), "silu_mul");
+                gemv(x2.p, w.w2, ffn_out, dim, hidden);
+            }
+            delta = ffn_out;
+        }
+        // final norm + classifier; the final hidden state must end in x
+        ck(tl_gemv_add_rms_norm_f16(h, delta, final_norm, eps, classifier, logits.p, h_other, vocab, dim),
+           "gemv_add_rms_norm");
+        std::swap(h, h_other);
+        if (h != x.p) ck(tl_memcpy_d2d(x.p, h, (size_t)dim * sizeof(half)), "memcpy_d2d");
+    }
+
+    // The same step with add + RMSNorm as launches of their own (hidden sizes the fused GEMV does not cover).
+    void decode_fused_separate_norm(int pos) {
         const int H = n_heads, D = head_dim;
         ck(tl_rms_norm_f16(x_norm.p, x.p, layers[0].att_norm, eps, dim, 1), "rms_norm");
         for (int l = 0; l < n_layers; ++l) {
@@ -202,6 +259,7 @@ struct tlm_model {
             const half* next_norm = (l + 1 < n_layers) ? layers[l + 1].att_norm : final_norm;
             ck(tl_add_rms_norm_f16(x.p, x_norm.p, x_residual.p, x.p, next_norm, eps, dim, 1), "add_rms_norm");
         }
+        gemv(x_norm.p, classifier, logits.p, vocab, dim);
     }
 
     half* forward(const int* dev_tokens, int S, int start_pos, int mode, bool all_logits) {
@@ -213,8 +271,7 @@ struct tlm_model {
         // the fused attention kernel covers head_dim 64/128/256; other sizes take the reference chain
         const bool fused_ok = head_dim == 64 || head_dim == 128 || head_dim == 256;
         if (mode == TLM_MODE_FUSED && S == 1 && fused_ok) {
-            decode_fused(start_pos);   // leaves rmsnorm(x) * final_norm in x_norm
-            gemv(x_norm.p, classifier, logits.p, vocab, dim);
+            decode_fused(start_pos);   // logits included
             return logits.p;
         }
         const bool use_mask = S > 1;   // get_mask: nullopt when seqlen <= 1   Transformer.cpp:234

@@ -271,6 +271,44 @@ def test_gemv_silu_mul(dev, oracle, N, K):
     assert np.array_equal(got.view(np.uint16), two.view(np.uint16))
 
 
+@pytest.mark.parametrize("N,K,with_addend", [(12288, 4096, True), (22016, 4096, True), (32000, 4096, True),
+                                             (300, 512, True), (64, 4096, False), (33, 11008, True), (10, 520, True)])
+def test_gemv_add_rms_norm(dev, oracle, N, K, with_addend):
+    """Residual add + RMSNorm formed inside the GEMV's operand load: against the CPU chain
+    (EwiseAdd -> RMSNorm -> matmul2d) and against the GPU's own three-step path."""
+    h = synth.normal_f16(150, (K,), 1.0)
+    d = synth.normal_f16(151, (K,), 0.7) if with_addend else None
+    g = synth.normal_f16(152, (K,), 1.0)
+    W = synth.normal_f16(153, (N, K), 0.02)
+    eps = 1e-5
+    want_sum = oracle.binary(h, d, "add") if with_addend else h
+    want_norm = oracle.rms_norm(want_sum[None, :], g, eps, "exact")[0]
+    want = oracle.matmul2d(want_norm[None, :], W)[0]
+    hd, gd, Wd = dev.from_numpy(h), dev.from_numpy(g), dev.from_numpy(W)
+    dd = dev.from_numpy(d) if with_addend else None
+    y, s = dev.gemv_add_rms_norm(hd, dd, gd, eps, Wd)
+    assert np.array_equal(s.cpu().numpy().view(np.uint16), want_sum.view(np.uint16))
+    # the norm is rounded from a differently ordered fp32 sum of squares: compare on the output scale
+    assert_close_scaled(y.cpu().numpy(), want, 1e-2, 5e-3, "gemv with fused add + rmsnorm")
+    if with_addend:
+        s2, n2 = dev.add_rms_norm(hd, dd, gd, eps)
+    else:
+        s2, n2 = hd, dev.rms_norm(hd.view(1, K), gd, eps).view(K)
+    two = dev.gemv(n2, Wd).cpu().numpy()
+    assert_close_scaled(y.cpu().numpy(), two, 1e-2, 2e-3, "fused vs three-step GPU path")
+    assert np.array_equal(hd.cpu().numpy().view(np.uint16), h.view(np.uint16))       # inputs untouched
+    y3, s3 = dev.gemv_add_rms_norm(hd, dd, gd, eps, Wd, want_sum=False)
+    assert s3 is None and np.array_equal(y3.cpu().numpy().view(np.uint16), y.cpu().numpy().view(np.uint16))
+
+
+def test_gemv_add_rms_norm_limits(dev):
+    from tensorlib_amd import TensorLibError
+    with pytest.raises(TensorLibError):
+        dev.gemv_add_rms_norm(dev.empty(16384), None, dev.empty(16384), 1e-5, dev.empty(8, 16384))  # K too long
+    with pytest.raises(TensorLibError):
+        dev.gemv_add_rms_norm(dev.empty(100), None, dev.empty(100), 1e-5, dev.empty(8, 100))        # K % 8 != 0
+
+
 def test_gemv_silu_mul_limits(dev):
     from tensorlib_amd import TensorLibError
     with pytest.raises(TensorLibError):
@@ -289,8 +327,8 @@ def test_rope_table_values(dev):
 
 
 def test_decode_attention_repeated_calls_reuse_counters(dev, oracle):
-    """The chunk-merge tickets must be back at zero after every launch: many calls in a row, with
-    different numbers of chunks, all have to agree with the CPU chain."""
+    """Many calls in a row with different numbers of chunks share one partials workspace: all of
+    them have to agree with the CPU chain."""
     H, D = 8, 128
     q = synth.normal_f16(140, (H, D), 1.0)
     ck = synth.normal_f16(141, (700, H, D), 1.0)
