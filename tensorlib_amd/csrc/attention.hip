@@ -216,7 +216,9 @@ decode_attn_partial_kernel(half_t* out, float* partial, const half_t* q, half_t*
 
 // Second pass: merge the chunk partials of one head.  (Folding this into the first launch with a
 // "last workgroup merges" ticket was measured slower: the device-scope fences it needs cost more
-// than this 4 us launch.)
+// than this 4 us launch.  So was one 1024-thread workgroup per head covering up to 512 positions
+// alone: 32 workgroups pull a context through 32 CUs' L2 ports instead of 256, and a whole decode
+// step lost 6 %.)
 __global__ void __launch_bounds__(256)
 decode_attn_merge_kernel(half_t* out, const float* partial, int D, int n_chunks) {
     const int h = blockIdx.x;
