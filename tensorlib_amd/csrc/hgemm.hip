@@ -622,20 +622,32 @@ static int hgemm_variant_index(const char* name) {
     return 1;
 }
 
-// Measured on MI355X over the Llama2-7B prefill shapes (M in {128,512,2048}):
-//   >= ~0.9 x CUs tiles of 256x256 : 256x256x64, 8 wavefronts (128x64 each), 2-stage LDS ring, fragments
-//                                    double buffered
-//   M >= 1024 otherwise            : 128x256x64, 8 wavefronts, fragments double buffered
-//   fewer rows                     : 128x128x64, 8 wavefronts, plus split-K (see launch_hgemm)
+// Measured on MI355X over the Llama2-7B prefill shapes (M in {128, 512, 1024, 2048}).
+// Up to 512 rows: 256x256x64 when its tiles nearly fill the chip, otherwise 128x128x64 plus split-K (see
+// launch_hgemm).  More rows: the tile shape with the cheapest schedule.  One round of 256x256 tiles on
+// every CU costs R; a round of 128x256 tiles (one workgroup per CU) or of 128x128 tiles (two per CU) does
+// half the work in 0.57 R (0.63 R), so the big tile wins unless its last round is mostly empty; a partly filled
+// round of a fraction f of the CUs costs about (0.65 + 0.3 f) of a full one (fewer busy CUs clock higher).
+// Splitting K or peeling the last round off into a second K-split launch lost to this on every shape tried.
 static int pick_variant(size_t M, size_t N, size_t K, int cus) {
     static const int v_big = hgemm_variant_index("p256x256x64w2x4s2");
     static const int v_mid = hgemm_variant_index("p128x256x64w2x4s2");
     static const int v_small = hgemm_variant_index("p128x128x64w2x4s2");
     (void)K;
     auto tiles = [&](int bm, int bn) { return ((M + bm - 1) / bm) * ((N + bn - 1) / bn); };
-    if (tiles(256, 256) * 10 >= (size_t)cus * 9) return v_big;
-    if (M >= 1024) return v_mid;
-    return v_small;
+    if (M <= 512) return tiles(256, 256) * 10 >= (size_t)cus * 9 ? v_big : v_small;
+    auto cost = [&](size_t t, size_t slots, double round_cost) {
+        const size_t full = t / slots, rem = t % slots;
+        return round_cost * ((double)full + (rem ? 0.65 + 0.3 * (double)rem / (double)slots : 0.0));
+    };
+    const double c_big = cost(tiles(256, 256), (size_t)cus, 1.0);
+    const double c_mid = cost(tiles(128, 256), (size_t)cus, 0.565);
+    const double c_small = cost(tiles(128, 128), (size_t)cus * 2, 0.63);
+    int best = v_big;
+    double c = c_big;
+    if (c_mid < c * 0.97) { best = v_mid; c = c_mid; }
+    if (c_small < c * 0.97) { best = v_small; c = c_small; }
+    return best;
 }
 
 int launch_hgemm(const void* A, const void* B, void* C, size_t M, size_t N, size_t K, size_t batch, size_t sa,
@@ -695,7 +707,9 @@ int launch_hgemm(const void* A, const void* B, void* C, size_t M, size_t N, size
         splits = g_forced_splits;
         if (splits <= 0) {
             // aim at ~1.5 workgroups per CU, keep at least 8 K tiles per split
-            splits = (int)(((size_t)cus * 3 / 2) / nblocks);
+            // (only for few rows: with more than 512 rows pick_variant already found a tile shape that
+            // fills the chip well enough, and splitting measured slower there)
+            splits = M <= 512 ? (int)(((size_t)cus * 3 / 2) / nblocks) : 1;
             const int max_by_k = KT / 8 > 0 ? KT / 8 : 1;
             if (splits > max_by_k) splits = max_by_k;
             if (splits > 16) splits = 16;
