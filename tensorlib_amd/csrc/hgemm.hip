@@ -376,9 +376,16 @@ __global__ void __launch_bounds__(WM* WN * 64) hgemm_f16_dlds_kernel(HgemmArgs a
                     issue_after_sync(kt + 1);
                     load_frags(af[nxt], bf[nxt], kt + 1, 0);
                 }
-                // keep the reads of the next step ahead of this step's MFMAs, so they land under them
-                __builtin_amdgcn_sched_barrier(0);
                 mfmas(af[cur], bf[cur]);
+                // Issue order inside the step: one fragment read of the next step behind each of the first
+                // MFMAs (an MFMA occupies the matrix core for 32 cycles but its issue slot for 4, so the reads
+                // go out under it and land under the rest of the step), nothing crosses into the next step.
+#pragma unroll
+                for (int r = 0; r < MT + NT; ++r) {
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // 1 MFMA
+                    __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // 1 LDS read
+                }
+                __builtin_amdgcn_sched_group_barrier(0x008, MT * NT - (MT + NT), 0);
                 __builtin_amdgcn_sched_barrier(0);
             }
         };
