@@ -585,6 +585,10 @@ static const HgemmVariant g_variants[] = {
     TL_HGEMM_PIPE(128, 256, 64, 2, 2, 2),  // 35
     TL_HGEMM_PIPE(128, 128, 64, 2, 4, 2),  // 36
     TL_HGEMM_PIPE(256, 256, 32, 2, 4, 4),  // 37
+    TL_HGEMM_PIPE(128, 64, 64, 2, 2, 4),   // 38  few rows: narrow B tiles, deep ring
+    TL_HGEMM_PIPE(128, 64, 64, 4, 1, 4),   // 39
+    TL_HGEMM_PIPE(128, 128, 64, 2, 4, 4),  // 40
+    TL_HGEMM_PIPE(256, 128, 64, 2, 4, 3),  // 41
 };
 static constexpr int kNumVariants = sizeof(g_variants) / sizeof(g_variants[0]);
 static int g_forced_variant = 0;
@@ -629,20 +633,31 @@ static int hgemm_variant_index(const char* name) {
     return 1;
 }
 
-// Measured on MI355X over the Llama2-7B prefill shapes (M in {128, 512, 1024, 2048}).
-// Up to 512 rows: 256x256x64 when its tiles nearly fill the chip, otherwise 128x128x64 plus split-K (see
-// launch_hgemm).  More rows: the tile shape with the cheapest schedule.  One round of 256x256 tiles on
-// every CU costs R; a round of 128x256 tiles (one workgroup per CU) or of 128x128 tiles (two per CU) does
-// half the work in 0.57 R (0.63 R), so the big tile wins unless its last round is mostly empty; a partly filled
-// round of a fraction f of the CUs costs about (0.65 + 0.3 f) of a full one (fewer busy CUs clock higher).
-// Splitting K or peeling the last round off into a second K-split launch lost to this on every shape tried.
+// Measured on MI355X over the Llama2-7B prefill shapes (M in {128, 512, 1024, 2048}), B streamed from HBM.
+// Up to 512 rows the problem is bound by streaming B once: the largest tile shape that still gives one
+// round of at least 0.6 x CUs workgroups, with a deep (3-4 stage) ring; if even 128x64 tiles are too few,
+// K is split until the chip is full (see launch_hgemm).
+// More rows: the tile shape with the cheapest schedule.  One round of 256x256 tiles on every CU costs R; a
+// round of 128x256 tiles (one workgroup per CU) or of 128x128 tiles (two per CU) does half the work in
+// 0.57 R (0.63 R), so the big tile wins unless its last round is mostly empty; a partly filled round of a
+// fraction f of the CUs costs about (0.65 + 0.3 f) of a full one (fewer busy CUs clock higher).  Splitting K
+// or peeling the last round off into a second K-split launch lost to this on every shape tried.
 static int pick_variant(size_t M, size_t N, size_t K, int cus) {
     static const int v_big = hgemm_variant_index("p256x256x64w2x4s2");
     static const int v_mid = hgemm_variant_index("p128x256x64w2x4s2");
     static const int v_small = hgemm_variant_index("p128x128x64w2x4s2");
-    (void)K;
+    static const int v_few_256x128 = hgemm_variant_index("p256x128x64w2x4s3");
+    static const int v_few_128x128 = hgemm_variant_index("p128x128x64w2x4s4");
+    static const int v_few_128x64 = hgemm_variant_index("p128x64x64w4x1s4");
     auto tiles = [&](int bm, int bn) { return ((M + bm - 1) / bm) * ((N + bn - 1) / bn); };
-    if (M <= 512) return tiles(256, 256) * 10 >= (size_t)cus * 9 ? v_big : v_small;
+    if (M <= 512 && tiles(256, 256) <= (size_t)cus) {
+        const size_t enough = (size_t)cus * 6 / 10;
+        if (tiles(256, 256) >= enough) return v_big;
+        if (M > 128 && tiles(256, 128) >= enough) return v_few_256x128;
+        // a long K can be halved instead of narrowing the tile
+        if (tiles(128, 128) >= enough || (K >= 8192 && tiles(128, 128) * 2 >= enough)) return v_few_128x128;
+        return v_few_128x64;
+    }
     auto cost = [&](size_t t, size_t slots, double round_cost) {
         const size_t full = t / slots, rem = t % slots;
         return round_cost * ((double)full + (rem ? 0.65 + 0.3 * (double)rem / (double)slots : 0.0));
@@ -713,10 +728,10 @@ int launch_hgemm(const void* A, const void* B, void* C, size_t M, size_t N, size
         const int cus = device_info().cu_count;
         splits = g_forced_splits;
         if (splits <= 0) {
-            // aim at ~1.5 workgroups per CU, keep at least 8 K tiles per split
+            // aim at one workgroup per CU, keep at least 8 K tiles per split
             // (only for few rows: with more than 512 rows pick_variant already found a tile shape that
             // fills the chip well enough, and splitting measured slower there)
-            splits = M <= 512 ? (int)(((size_t)cus * 3 / 2) / nblocks) : 1;
+            splits = M <= 512 ? (int)((size_t)cus / nblocks) : 1;
             const int max_by_k = KT / 8 > 0 ? KT / 8 : 1;
             if (splits > max_by_k) splits = max_by_k;
             if (splits > 16) splits = 16;
