@@ -220,6 +220,24 @@ int tl_rope_qk_store_kv_f16(void* qkv, void* cache_k, void* cache_v, int pos, in
 int tl_add_rms_norm_f16(void* sum_out, void* norm_out, const void* a, const void* b, const void* weight,
                         float eps, int hidden_size, int num_tokens);
 
+/* Prefill glue after the q, k, v projections of n_tokens rows with row stride `row_stride` elements
+ * (dim, or 3*dim for one fused q|k|v GEMM): q is rotated and written head-major [n_heads, n_tokens,
+ * head_dim], k is rotated into cache_k[start_pos + s], v copied into cache_v[start_pos + s].  Replaces two
+ * apply_rotary_emb, two setItem and one transpose+contiguous of Attention::forward
+ * (model/llama2_7b/src/Transformer.cpp:47-60).  rope_table as built by tl_rope_table_f16. */
+int tl_prefill_rope_qkv_f16(void* q_out, const void* q, const void* k, const void* v, size_t row_stride,
+                            void* cache_k, void* cache_v, const void* rope_table, int start_pos, int n_tokens,
+                            int n_heads, int head_dim);
+
+/* In place on scores [n_heads, seqlen, start_pos + seqlen]: ScalarDiv by `divisor` (fp16 bits), the causal
+ * mask add and softmax(3) of Attention::forward (model/llama2_7b/src/Transformer.cpp:94-105) in one launch;
+ * the quotient is rounded to fp16 before the softmax, as the separate kernels store it. */
+int tl_scaled_causal_softmax_f16(void* scores, uint16_t divisor_bits, int n_heads, int seqlen, int start_pos);
+
+/* out[r, j] = silu(ab[r, j]) * ab[r, hidden + j] for rows of a fused w1|w3 projection [rows, 2*hidden]
+ * (FeedForward::forward, model/llama2_7b/src/Transformer.cpp:137-141).  hidden % 8 == 0. */
+int tl_silu_mul_rows_f16(void* out, const void* ab, size_t rows, size_t hidden);
+
 /* mask[r,i,j] = (j > start_pos + i) ? -inf : 0 for r < reps, i < seqlen, j < start_pos+seqlen.
  * Replaces the element-by-element host loop of Transformer::get_mask
  * (model/llama2_7b/src/Transformer.cpp:231-261). */

@@ -249,6 +249,35 @@ causal_mask_kernel(half_t* mask, int seqlen, int start_pos, size_t n) {
     }
 }
 
+// Prefill glue after the q, k, v projections of n_tokens rows (row stride `ld`, e.g. 3*dim for a fused
+// q|k|v GEMM): one thread per (token, head, pair).  q is rotated and written head-major [H, S, D] (the
+// layout the per-head score matmul wants), k is rotated into cache_k[start_pos + s], v copied into cache_v.
+// Same arithmetic as rope_kernel with the table's half-rounded cos/sin.
+__global__ void __launch_bounds__(256)
+prefill_rope_qkv_kernel(half_t* q_out, const half_t* q, const half_t* k, const half_t* v, size_t ld, half_t* cache_k,
+                        half_t* cache_v, const half_t* rope_table, int start_pos, int n_tokens, int n_heads,
+                        int head_dim) {
+    const int half_d = head_dim / 2;
+    const size_t total = (size_t)n_tokens * n_heads * half_d;
+    const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= total) return;
+    const int pair = (int)(idx % half_d);
+    const int h = (int)((idx / half_d) % n_heads);
+    const int s = (int)(idx / ((size_t)half_d * n_heads));
+    const half2_t cs = *reinterpret_cast<const half2_t*>(rope_table + ((size_t)(start_pos + s) * half_d + pair) * 2);
+    const float c = (float)cs[0], sn = (float)cs[1];
+    const size_t in_off = (size_t)s * ld + (size_t)h * head_dim + 2 * pair;
+    const half2_t qv = *reinterpret_cast<const half2_t*>(q + in_off);
+    const half2_t kv = *reinterpret_cast<const half2_t*>(k + in_off);
+    const half2_t vv = *reinterpret_cast<const half2_t*>(v + in_off);
+    half2_t qr = {(half_t)((float)qv[0] * c - (float)qv[1] * sn), (half_t)((float)qv[0] * sn + (float)qv[1] * c)};
+    half2_t kr = {(half_t)((float)kv[0] * c - (float)kv[1] * sn), (half_t)((float)kv[0] * sn + (float)kv[1] * c)};
+    *reinterpret_cast<half2_t*>(q_out + ((size_t)h * n_tokens + s) * head_dim + 2 * pair) = qr;
+    const size_t c_off = ((size_t)(start_pos + s) * n_heads + h) * head_dim + 2 * pair;
+    *reinterpret_cast<half2_t*>(cache_k + c_off) = kr;
+    *reinterpret_cast<half2_t*>(cache_v + c_off) = vv;
+}
+
 // Decode-step glue after the fused q|k|v GEMV: rotate q in place, rotate k and write it to
 // cache_k[pos], copy v to cache_v[pos].  One thread per (even, odd) pair of the 3*dim vector.
 __global__ void __launch_bounds__(256)
@@ -456,6 +485,29 @@ int tl_rope_table_f16(void* table, int max_seq, int head_dim) {
     hipLaunchKernelGGL(tl::rope_table_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, tl::stream(),
                        (tl::half_t*)table, max_seq, head_dim);
     TL_CHECK_LAUNCH("rope_table_kernel");
+    return TL_OK;
+}
+
+int tl_prefill_rope_qkv_f16(void* q_out, const void* q, const void* k, const void* v, size_t row_stride, void* cache_k,
+                            void* cache_v, const void* rope_table, int start_pos, int n_tokens, int n_heads,
+                            int head_dim) {
+    TL_ENSURE_INIT();
+    TL_REQUIRE(q_out && q && k && v && cache_k && cache_v && rope_table, "tl_prefill_rope_qkv_f16: null pointer");
+    TL_REQUIRE(start_pos >= 0 && n_tokens >= 0 && n_heads >= 1 && head_dim >= 2 && head_dim % 2 == 0,
+               "tl_prefill_rope_qkv_f16: bad sizes");
+    TL_REQUIRE(row_stride % 2 == 0 && row_stride >= (size_t)n_heads * head_dim,
+               "tl_prefill_rope_qkv_f16: row stride %zu too small or odd", row_stride);
+    auto al4 = [](const void* p) { return ((uintptr_t)p & 3) == 0; };
+    TL_REQUIRE(al4(q_out) && al4(q) && al4(k) && al4(v) && al4(cache_k) && al4(cache_v) && al4(rope_table),
+               "tl_prefill_rope_qkv_f16: pointers must be 4-byte aligned");
+    const size_t total = (size_t)n_tokens * n_heads * (head_dim / 2);
+    if (total == 0) return TL_OK;
+    TL_REQUIRE((total + 255) / 256 <= 0x7fffffffu, "tl_prefill_rope_qkv_f16: too many elements");
+    hipLaunchKernelGGL(tl::prefill_rope_qkv_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, tl::stream(),
+                       (tl::half_t*)q_out, (const tl::half_t*)q, (const tl::half_t*)k, (const tl::half_t*)v, row_stride,
+                       (tl::half_t*)cache_k, (tl::half_t*)cache_v, (const tl::half_t*)rope_table, start_pos, n_tokens,
+                       n_heads, head_dim);
+    TL_CHECK_LAUNCH("prefill_rope_qkv_kernel");
     return TL_OK;
 }
 

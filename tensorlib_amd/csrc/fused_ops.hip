@@ -2,6 +2,8 @@
 // leaves the GPU: RMSNorm, RoPE, softmax, SiLU, elementwise add/sub/mul/div, strided
 // gather/scatter (contiguous / setItemEwise), argmax, embedding lookup, fill.
 // All HBM-trivial; written for 64-lane wavefronts with 16-byte accesses where alignment allows.
+#include <cstring>
+
 #include "tl_internal.h"
 
 namespace tl {
@@ -153,6 +155,43 @@ struct AddOp { __device__ static half_t apply(half_t a, half_t b) { return (half
 struct SubOp { __device__ static half_t apply(half_t a, half_t b) { return (half_t)((float)a - (float)b); } };
 struct MulOp { __device__ static half_t apply(half_t a, half_t b) { return (half_t)((float)a * (float)b); } };
 struct DivOp { __device__ static half_t apply(half_t a, half_t b) { return (half_t)((float)a / (float)b); } };
+
+// In-place softmax over rows of attention scores with the two elementwise steps that precede it in
+// Attention::forward folded into the load: v = half(x / divisor) (ScalarDiv), columns beyond
+// start_pos + (row % seqlen) are -inf (the causal mask EwiseAdd would have made them -inf).  The values
+// entering the softmax are the same halves the three-kernel chain would have read.
+__global__ void __launch_bounds__(256)
+scaled_causal_softmax_kernel(half_t* scores, half_t divisor, int seqlen, int start_pos, size_t cols) {
+    __shared__ float red[16];
+    half_t* x = scores + (size_t)blockIdx.x * cols;
+    const size_t limit = (size_t)start_pos + (blockIdx.x % (unsigned)seqlen);  // last visible column
+    const float d = (float)divisor;
+    auto val = [&](size_t j) { return j <= limit ? (float)(half_t)((float)x[j] / d) : -INFINITY; };
+    float mx = -INFINITY;
+    for (size_t j = threadIdx.x; j < cols; j += blockDim.x) mx = fmaxf(mx, val(j));
+    mx = block_max_f(mx, red);
+    float sum = 0.f;
+    for (size_t j = threadIdx.x; j < cols; j += blockDim.x) sum += expf(val(j) - mx);
+    sum = block_sum_f(sum, red);
+    const float inv = 1.0f / sum;
+    for (size_t j = threadIdx.x; j < cols; j += blockDim.x) x[j] = (half_t)(expf(val(j) - mx) * inv);
+}
+
+// out[r][j] = silu(ab[r][j]) * ab[r][hidden + j]: SwiGLU gate on the rows of a fused w1|w3 projection.
+__global__ void __launch_bounds__(256)
+silu_mul_rows_kernel(half_t* out, const half_t* ab, int hidden, size_t n8) {
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    const size_t h8 = (size_t)hidden / 8;
+    for (size_t c = (size_t)blockIdx.x * blockDim.x + threadIdx.x; c < n8; c += stride) {
+        const size_t r = c / h8, j = c % h8;
+        const half8_t va = reinterpret_cast<const half8_t*>(ab)[r * 2 * h8 + j];
+        const half8_t vb = reinterpret_cast<const half8_t*>(ab)[r * 2 * h8 + h8 + j];
+        half8_t o;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) o[e] = SiluMulOp::apply(va[e], vb[e]);
+        reinterpret_cast<half8_t*>(out)[c] = o;
+    }
+}
 
 // out[i] = Op(a[i], b[i])  (B_MODE 0: no second operand, 1: tensor, 2: scalar)
 template <typename Op, int B_MODE, bool VEC>
@@ -407,6 +446,38 @@ int tl_softmax_f16(void* out, const void* in, size_t rows, size_t cols) {
     hipLaunchKernelGGL(tl::softmax_kernel, dim3((unsigned)rows), dim3(threads), 0, tl::stream(), (tl::half_t*)out,
                        (const tl::half_t*)in, cols);
     TL_CHECK_LAUNCH("softmax_kernel");
+    return TL_OK;
+}
+
+int tl_scaled_causal_softmax_f16(void* scores, uint16_t divisor_bits, int n_heads, int seqlen, int start_pos) {
+    TL_ENSURE_INIT();
+    TL_REQUIRE(n_heads >= 0 && seqlen >= 0 && start_pos >= 0, "tl_scaled_causal_softmax_f16: negative size");
+    const size_t rows = (size_t)n_heads * seqlen, cols = (size_t)start_pos + seqlen;
+    if (rows == 0) return TL_OK;
+    TL_REQUIRE(scores, "tl_scaled_causal_softmax_f16: null pointer");
+    TL_REQUIRE(rows <= 0x7fffffffu, "tl_scaled_causal_softmax_f16: too many rows (%zu)", rows);
+    tl::half_t d;
+    memcpy(&d, &divisor_bits, 2);
+    const int threads = cols <= 64 ? 64 : cols <= 128 ? 128 : 256;
+    hipLaunchKernelGGL(tl::scaled_causal_softmax_kernel, dim3((unsigned)rows), dim3(threads), 0, tl::stream(),
+                       (tl::half_t*)scores, d, seqlen, start_pos, cols);
+    TL_CHECK_LAUNCH("scaled_causal_softmax_kernel");
+    return TL_OK;
+}
+
+int tl_silu_mul_rows_f16(void* out, const void* ab, size_t rows, size_t hidden) {
+    TL_ENSURE_INIT();
+    if (rows == 0 || hidden == 0) return TL_OK;
+    TL_REQUIRE(out && ab, "tl_silu_mul_rows_f16: null pointer");
+    TL_REQUIRE(hidden % 8 == 0 && hidden <= 0x7fffffffu && tl::aligned16(out) && tl::aligned16(ab),
+               "tl_silu_mul_rows_f16: needs hidden %% 8 == 0 and 16-byte aligned operands");
+    const size_t n8 = rows * hidden / 8;
+    size_t blocks = (n8 + 255) / 256;
+    const size_t cap = (size_t)tl::device_info().cu_count * 16;
+    if (blocks > cap) blocks = cap;
+    hipLaunchKernelGGL(tl::silu_mul_rows_kernel, dim3((unsigned)blocks), dim3(256), 0, tl::stream(), (tl::half_t*)out,
+                       (const tl::half_t*)ab, (int)hidden, n8);
+    TL_CHECK_LAUNCH("silu_mul_rows_kernel");
     return TL_OK;
 }
 

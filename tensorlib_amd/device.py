@@ -352,6 +352,43 @@ class HipDevice:
               "tl_gemv_add_rms_norm_f16")
         return y, s
 
+    def prefill_rope_qkv(self, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, cache_k: torch.Tensor,
+                         cache_v: torch.Tensor, table: torch.Tensor, start_pos: int, n_heads: int) -> torch.Tensor:
+        """q, k, v: [S, n_heads*head_dim] views sharing one row stride (e.g. column blocks of a fused
+        [S, 3*dim] projection).  Returns rotated q as [n_heads, S, head_dim]; rotated k and v go into
+        cache rows [start_pos, start_pos + S)."""
+        for t, nm in ((q, "q"), (k, "k"), (v, "v")):
+            if t.dtype != torch.float16 or not t.is_cuda or t.dim() != 2 or t.stride(1) != 1:
+                raise ValueError(f"{nm} must be a 2-D fp16 device tensor with unit column stride")
+        S, dim = q.shape
+        ld = q.stride(0)
+        if k.stride(0) != ld or v.stride(0) != ld or k.shape != q.shape or v.shape != q.shape:
+            raise ValueError("q, k, v must share shape and row stride")
+        D = dim // n_heads
+        out = torch.empty((n_heads, S, D), dtype=torch.float16, device=q.device)
+        check(self.lib.tl_prefill_rope_qkv_f16(_ptr(out), q.data_ptr(), k.data_ptr(), v.data_ptr(), ld, _ptr(cache_k),
+                                               _ptr(cache_v), _ptr(table), start_pos, S, n_heads, D),
+              "tl_prefill_rope_qkv_f16")
+        return out
+
+    def scaled_causal_softmax(self, scores: torch.Tensor, divisor: float, start_pos: int) -> torch.Tensor:
+        """In place on scores [n_heads, S, start_pos + S]: divide by half(divisor), causal mask, softmax."""
+        _req(scores, name="scores")
+        H, S, T = scores.shape
+        if T != start_pos + S:
+            raise ValueError("scores must be [n_heads, S, start_pos + S]")
+        bits = int(np.array(divisor, dtype=np.float16).view(np.uint16))
+        check(self.lib.tl_scaled_causal_softmax_f16(_ptr(scores), bits, H, S, start_pos), "tl_scaled_causal_softmax_f16")
+        return scores
+
+    def silu_mul_rows(self, ab: torch.Tensor) -> torch.Tensor:
+        """ab: [rows, 2*hidden] -> silu(ab[:, :hidden]) * ab[:, hidden:]."""
+        _req(ab, name="ab")
+        rows, two_h = ab.shape
+        out = torch.empty((rows, two_h // 2), dtype=torch.float16, device=ab.device)
+        check(self.lib.tl_silu_mul_rows_f16(_ptr(out), _ptr(ab), rows, two_h // 2), "tl_silu_mul_rows_f16")
+        return out
+
     # -- tuning hooks -------------------------------------------------------------------
     def set_gemv_variant(self, v: int) -> None:
         check(self.lib.tl_set_gemv_variant(v), "tl_set_gemv_variant")

@@ -262,6 +262,57 @@ struct tlm_model {
         gemv(x_norm.p, classifier, logits.p, vocab, dim);
     }
 
+    // Prefill of S > 1 tokens with the glue ops fused: one q|k|v GEMM and one w1|w3 GEMM when the weights
+    // are adjacent, RoPE + cache write + q transpose in one launch, ScalarDiv + mask + softmax in one launch,
+    // residual add + RMSNorm in one launch, SwiGLU gate in one launch.  14 launches per layer instead of 27;
+    // the matmuls are the same calls as in the reference chain.  Leaves rmsnorm(x) * final_norm in x_norm.
+    void prefill_fused(int S, int start_pos) {
+        const int T = start_pos + S, H = n_heads, D = head_dim;
+        const size_t sd = (size_t)S * dim;
+        union { half h; uint16_t u; } sq;
+        sq.h = (half)std::sqrt((float)D);
+        ck(tl_rms_norm_f16(x_norm.p, x.p, layers[0].att_norm, eps, dim, S), "rms_norm");
+        for (int l = 0; l < n_layers; ++l) {
+            const LayerWeights& w = layers[l];
+            const size_t dd = (size_t)dim * dim;
+            const half *q, *k, *v;
+            size_t ld;
+            if (w.wk == w.wq + dd && w.wv == w.wk + dd) {
+                matmul2d(x_norm.p, w.wq, qkv.p, S, (size_t)3 * dim, dim);   // rows of q | k | v
+                q = qkv.p; k = qkv.p + dim; v = qkv.p + 2 * dim; ld = (size_t)3 * dim;
+            } else {
+                matmul2d(x_norm.p, w.wq, xq(S), S, dim, dim);
+                matmul2d(x_norm.p, w.wk, xk(S), S, dim, dim);
+                matmul2d(x_norm.p, w.wv, xv(S), S, dim, dim);
+                q = xq(S); k = xk(S); v = xv(S); ld = dim;
+            }
+            ck(tl_prefill_rope_qkv_f16(xq_c.p, q, k, v, ld, cache_k[l].p, cache_v[l].p, rope_table.p, start_pos, S, H, D),
+               "prefill_rope_qkv");
+            // keys -> [H,T,D], values -> [H,D,T] (what the per-head matmul2d calls consume)   Transformer.cpp:61-80
+            cache_k[l].dev->contiguous(keys_c.p, {1, H, T, D}, {max_seq * dim, D, dim, 1}, 0, (size_t)T * dim);
+            cache_v[l].dev->contiguous(values_c.p, {1, H, D, T}, {max_seq * dim, D, 1, dim}, 0, (size_t)T * dim);
+            ck(tl_matmul2d_batched_f16(xq_c.p, keys_c.p, scores.p, S, T, D, H, (size_t)S * D, (size_t)T * D, (size_t)S * T),
+               "scores");
+            ck(tl_scaled_causal_softmax_f16(scores.p, sq.u, H, S, start_pos), "scaled_causal_softmax");
+            ck(tl_matmul2d_batched_f16(scores.p, values_c.p, s_v.p, S, D, T, H, (size_t)S * T, (size_t)D * T, (size_t)S * D),
+               "scores.values");
+            s_v.dev->contiguous(o_c.p, {1, S, H, D}, {H * S * D, D, S * D, 1}, 0, sd);
+            matmul2d(o_c.p, w.wo, x_norm.p, S, dim, dim);
+            ck(tl_add_rms_norm_f16(x_residual.p, x_norm.p, x.p, x_norm.p, w.ffn_norm, eps, dim, S), "add_rms_norm");
+            if (w.w3 == w.w1 + (size_t)hidden * dim && hidden % 8 == 0) {
+                matmul2d(x_norm.p, w.w1, x13.p, S, (size_t)2 * hidden, dim);   // rows of w1.x | w3.x
+                ck(tl_silu_mul_rows_f16(x2.p, x13.p, S, hidden), "silu_mul_rows");
+            } else {
+                matmul2d(x_norm.p, w.w1, x1(S), S, hidden, dim);
+                matmul2d(x_norm.p, w.w3, x3(S), S, hidden, dim);
+                ck(tl_silu_mul_f16(x2.p, x1(S), x3(S), (size_t)S * hidden), "silu_mul");
+            }
+            matmul2d(x2.p, w.w2, x.p, S, dim, hidden);
+            const half* next_norm = (l + 1 < n_layers) ? layers[l + 1].att_norm : final_norm;
+            ck(tl_add_rms_norm_f16(x.p, x_norm.p, x_residual.p, x.p, next_norm, eps, dim, S), "add_rms_norm");
+        }
+    }
+
     half* forward(const int* dev_tokens, int S, int start_pos, int mode, bool all_logits) {
         check_weights();
         if (S < 1 || S > max_tokens) throw std::runtime_error("n_tokens out of range [1, max_tokens]");
@@ -272,6 +323,15 @@ struct tlm_model {
         const bool fused_ok = head_dim == 64 || head_dim == 128 || head_dim == 256;
         if (mode == TLM_MODE_FUSED && S == 1 && fused_ok) {
             decode_fused(start_pos);   // logits included
+            return logits.p;
+        }
+        if (mode == TLM_MODE_FUSED && S > 1) {
+            prefill_fused(S, start_pos);
+            if (all_logits) {
+                matmul2d(x_norm.p, classifier, logits.p, S, vocab, dim);
+            } else {
+                gemv(x_norm.p + (size_t)(S - 1) * dim, classifier, logits.p, vocab, dim);
+            }
             return logits.p;
         }
         const bool use_mask = S > 1;   // get_mask: nullopt when seqlen <= 1   Transformer.cpp:234

@@ -122,12 +122,15 @@ def test_llama2_7b_block_decode_kv1024_and_prefill_512(dev):
     toks = synth.token_ids(8, 512, cfg.vocab_size)
     ref = _oracle_model(cfg, w)
     ref.forward(toks, 0)
-    m = Llama2Model(dev, cfg, max_tokens=512)
-    m.set_weights(w)
-    m.forward(toks, 0, MODE_REFERENCE_CHAIN, all_logits=False)
-    got_x = m.get_buffer(BUF_X, 0, (512, cfg.dim)).cpu().numpy()
-    assert_close_scaled(got_x, ref.last_hidden, 1e-2, 1e-2, "block prefill hidden state")
-    m.close()
+    for mode in (MODE_REFERENCE_CHAIN, MODE_FUSED):
+        m = Llama2Model(dev, cfg, max_tokens=512)
+        m.set_weights(w)
+        m.forward(toks, 0, mode, all_logits=False)
+        got_x = m.get_buffer(BUF_X, 0, (512, cfg.dim)).cpu().numpy()
+        assert_close_scaled(got_x, ref.last_hidden, 1e-2, 1e-2, f"block prefill hidden state mode {mode}")
+        gk = m.get_buffer(BUF_CACHE_K, 0, (512, 32, 128)).cpu().numpy()
+        assert_close_scaled(gk, ref.cache_k[0][:512], 1e-2, 1e-2, f"block prefill cache_k mode {mode}")
+        m.close()
 
 
 def test_llama2_7b_full_model(dev):
@@ -151,6 +154,8 @@ def test_llama2_7b_full_model(dev):
         assert nrmse <= 1e-2 and worst <= 6e-2, (what, nrmse, worst)
 
     want_prefill = ref.forward(toks[:4], 0)
+    got = m.forward(toks[:4], 0, MODE_FUSED, all_logits=True).cpu().numpy()
+    check(got, want_prefill, "7B prefill logits (fused)")
     got = m.forward(toks[:4], 0, MODE_REFERENCE_CHAIN, all_logits=True).cpu().numpy()
     check(got, want_prefill, "7B prefill logits (chain)")
     for pos in (4, 5):
@@ -163,7 +168,10 @@ def test_llama2_7b_full_model(dev):
     out_f, tp_f, td_f = m.generate(prompt, 256, MODE_FUSED)
     out_c, tp_c, td_c = m.generate(prompt, 256, MODE_REFERENCE_CHAIN)
     assert out_f.min() >= 0 and out_f.max() < cfg.vocab_size and out_c.min() >= 0 and out_c.max() < cfg.vocab_size
-    assert out_f[0] == out_c[0]  # the first token comes from the same (chain) prefill path in both modes
+    # the two prefill paths differ only by fp16-rounding-level effects (different GEMM tilings)
+    lf = m.forward(prompt, 0, MODE_FUSED).cpu().numpy()
+    lc = m.forward(prompt, 0, MODE_REFERENCE_CHAIN).cpu().numpy()
+    check(lf, lc, "7B 128-token prefill logits, fused vs chain")
     # determinism: the same call twice gives the same tokens
     out_f2, _, _ = m.generate(prompt, 256, MODE_FUSED)
     assert np.array_equal(out_f, out_f2)

@@ -337,3 +337,68 @@ def test_decode_attention_repeated_calls_reuse_counters(dev, oracle):
     for T in (700, 65, 700, 130, 64, 129, 700):
         got = dev.decode_attention(qd, kd, vd, T).cpu().numpy()
         assert_close_f16(got, _attention_chain_oracle(oracle, q, ck, cv, T), RTOL, 2e-3, f"repeat T={T}")
+
+
+# ------------------------------------------------------------------- prefill glue ----
+
+@pytest.mark.parametrize("S,H,D,start,fused_rows", [(128, 32, 128, 0, True), (17, 4, 64, 5, False), (3, 2, 256, 40, True)])
+def test_prefill_rope_qkv(dev, oracle, S, H, D, start, fused_rows):
+    """RoPE of q and k, cache writes and the q transpose in one launch, from separate projections or
+    from the column blocks of one fused [S, 3*dim] projection."""
+    dim = H * D
+    qkv = synth.normal_f16(160, (S, 3 * dim), 1.0)
+    q, k, v = qkv[:, :dim], qkv[:, dim:2 * dim], qkv[:, 2 * dim:]
+    T = start + S + 2
+    ck0 = synth.normal_f16(161, (T, H, D), 1.0)
+    cv0 = synth.normal_f16(162, (T, H, D), 1.0)
+    want_q = oracle.rope(np.ascontiguousarray(q).reshape(1, S, H, D), start)[0]      # [S, H, D]
+    want_k = oracle.rope(np.ascontiguousarray(k).reshape(1, S, H, D), start)[0]
+    kd, vd = dev.from_numpy(ck0), dev.from_numpy(cv0)
+    table = dev.rope_table(T, D)
+    if fused_rows:
+        t = dev.from_numpy(qkv)
+        qd, kk, vv = t[:, :dim], t[:, dim:2 * dim], t[:, 2 * dim:]
+    else:
+        qd, kk, vv = (dev.from_numpy(np.ascontiguousarray(a)) for a in (q, k, v))
+    got_q = dev.prefill_rope_qkv(qd, kk, vv, kd, vd, table, start, H).cpu().numpy()   # [H, S, D]
+    assert_close_f16(got_q, want_q.transpose(1, 0, 2), RTOL, 2e-3, "prefill rope q")
+    gk, gv = kd.cpu().numpy(), vd.cpu().numpy()
+    assert_close_f16(gk[start:start + S], want_k, RTOL, 2e-3, "prefill rope k -> cache")
+    assert np.array_equal(gv[start:start + S].view(np.uint16), np.ascontiguousarray(v).reshape(S, H, D).view(np.uint16))
+    keep = np.r_[0:start, start + S:T]                                                   # other cache rows untouched
+    assert np.array_equal(gk[keep].view(np.uint16), ck0[keep].view(np.uint16))
+    assert np.array_equal(gv[keep].view(np.uint16), cv0[keep].view(np.uint16))
+    # identical bits to the per-op GPU path (apply_rotary_emb with the same half-rounded cos/sin)
+    q4 = dev.from_numpy(np.ascontiguousarray(q).reshape(1, S, H, D))
+    two = dev.apply_rotary_emb(q4, start).cpu().numpy()[0].transpose(1, 0, 2)
+    assert np.array_equal(got_q.view(np.uint16), two.view(np.uint16))
+
+
+@pytest.mark.parametrize("H,S,start", [(32, 128, 0), (4, 17, 9), (2, 1, 300), (3, 70, 0)])
+def test_scaled_causal_softmax(dev, oracle, H, S, start):
+    """ScalarDiv, mask add and softmax of Attention::forward in one launch, against the three CPU ops."""
+    T = start + S
+    sc = synth.normal_f16(170, (H, S, T), 8.0)
+    div = np.float16(np.sqrt(128.0))
+    t = oracle.binary_scalar(sc, div, "div")
+    mask = np.where(np.arange(T)[None, :] > start + np.arange(S)[:, None], -np.inf, 0.0).astype(np.float16)
+    t = oracle.binary(t, np.broadcast_to(mask, (H, S, T)).copy(), "add")
+    want = oracle.softmax(t.reshape(H * S, T)).reshape(H, S, T)
+    got = dev.scaled_causal_softmax(dev.from_numpy(sc), float(div), start).cpu().numpy()
+    assert_close_f16(got, want, RTOL, ATOL, "scaled causal softmax")
+    assert np.all(got[:, np.arange(S)[:, None] + start < np.arange(T)[None, :]] == 0)   # masked columns are exactly 0
+    # identical bits to the GPU's three-launch path
+    d3 = dev.binary(dev.from_numpy(sc), float(div), "div")
+    d3 = dev.binary(d3, dev.causal_mask(H, S, start).view(H, S, T), "add")
+    three = dev.softmax(d3.view(H * S, T)).cpu().numpy().reshape(H, S, T)
+    assert np.array_equal(got.view(np.uint16), three.view(np.uint16))
+
+
+@pytest.mark.parametrize("rows,hidden", [(128, 11008), (3, 64), (1, 8)])
+def test_silu_mul_rows(dev, oracle, rows, hidden):
+    ab = synth.normal_f16(180, (rows, 2 * hidden), 1.5)
+    want = oracle.silu_mul(np.ascontiguousarray(ab[:, :hidden]), np.ascontiguousarray(ab[:, hidden:]))
+    got = dev.silu_mul_rows(dev.from_numpy(ab)).cpu().numpy()
+    assert_close_f16(got, want, RTOL, ATOL, "silu_mul_rows")
+    two = dev.silu_mul(dev.from_numpy(np.ascontiguousarray(ab[:, :hidden])), dev.from_numpy(np.ascontiguousarray(ab[:, hidden:])))
+    assert np.array_equal(got.view(np.uint16), two.cpu().numpy().view(np.uint16))
