@@ -292,6 +292,14 @@ __global__ void __launch_bounds__(WM* WN * 64) hgemm_f16_dlds_kernel(HgemmArgs a
         for (int j = 0; j < B_LOADS; ++j)
             load_16B_per_lane_to_lds(b_src[j] + koff, sb + (j * NW + wave) * 1024);
     };
+    // wavefront-load l of tile kt: l < A_LOADS from A, the rest from B
+    auto issue_one = [&](int kt, int l) {
+        const size_t koff = (size_t)kt * BK;
+        if (l < A_LOADS)
+            load_16B_per_lane_to_lds(a_src[l] + koff, lds + a_off(kt) + (l * NW + wave) * 1024);
+        else
+            load_16B_per_lane_to_lds(b_src[l - A_LOADS] + koff, lds + b_off(kt) + ((l - A_LOADS) * NW + wave) * 1024);
+    };
 
     // ---- fragment reader: row (lane % 32) of a 32-row MFMA tile, chunk 2*ks + lane/32 ----
     const int fr_row = lane & 31;
@@ -372,9 +380,30 @@ __global__ void __launch_bounds__(WM* WN * 64) hgemm_f16_dlds_kernel(HgemmArgs a
                 if (ks + 1 < KS) {
                     load_frags(af[nxt], bf[nxt], kt, ks + 1);
                 } else if constexpr (decltype(has_next)::value) {
+                    // Last step of the tile: after the barrier the matrix core restarts at once, and the
+                    // requests for the tile after next and the first fragment reads of the next tile go out
+                    // one by one behind the MFMAs instead of in a block in front of them.
                     sync_for(kt + 1);  // every wavefront holds its last fragments of tile kt in registers
-                    issue_after_sync(kt + 1);
-                    load_frags(af[nxt], bf[nxt], kt + 1, 0);
+                    const bool more = kt + STAGES < KT;
+                    constexpr int NM = MT * NT;
+                    const unsigned char* sa = smem_raw + a_off(kt + 1) + a_base;
+                    const unsigned char* sb = smem_raw + b_off(kt + 1) + b_base;
+#pragma unroll
+                    for (int m = 0; m < NM; ++m) {
+                        const int i = m / NT, j = m % NT;
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(bf[cur][j], af[cur][i], acc[i][j], 0, 0, 0);
+#pragma unroll
+                        for (int r = m; r < MT + NT; r += NM) {
+                            if (r < MT) af[nxt][r] = *reinterpret_cast<const half8_t*>(sa + r * 32 * RB + fr_off[0]);
+                            else bf[nxt][r - MT] = *reinterpret_cast<const half8_t*>(sb + (r - MT) * 32 * RB + fr_off[0]);
+                        }
+                        if (more) {
+#pragma unroll
+                            for (int l = m; l < LPW; l += NM) issue_one(kt + STAGES, l);
+                        }
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
+                    continue;
                 }
                 mfmas(af[cur], bf[cur]);
                 // Issue order inside the step: one fragment read of the next step behind each of the first
