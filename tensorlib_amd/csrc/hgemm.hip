@@ -231,6 +231,11 @@ __global__ void __launch_bounds__(WM* WN * 64) hgemm_f16_dlds_kernel(HgemmArgs a
     static_assert(BK == 32 || BK == 64, "BK must be 32 or 64");
     static_assert(BM % (RPW * NW) == 0 && BN % (RPW * NW) == 0, "tile rows must split over the wavefronts");
     static_assert(STAGES >= 2 && STAGES <= 5 && LPW * (STAGES - 2) < 64, "vmcnt is a 6-bit counter");
+    // Two-stage pipelined variants are persistent: a workgroup walks tiles blockIdx.x, + gridDim.x, ... and
+    // requests the first K tile of its next C tile before it stores the current one, so the C stores and
+    // the cold start of the next tile overlap.  (vmcnt counts loads and stores together on this ISA, which
+    // is fine for two stages: every tile barrier waits for vmcnt(0) anyway.)
+    constexpr bool PERSIST = (STAGES == 2 && MODE == 1);
 
     extern __shared__ __attribute__((aligned(1024))) unsigned char smem_raw[];
     typedef __attribute__((address_space(3))) unsigned char lds_byte_t;
@@ -241,9 +246,8 @@ __global__ void __launch_bounds__(WM* WN * 64) hgemm_f16_dlds_kernel(HgemmArgs a
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave / WN, wn = wave % WN;
 
-    int tile_m, tile_n;
-    tile_of_block(blockIdx.x, gridDim.x, a.tiles_m, tile_m, tile_n);
-    const int m0 = tile_m * BM, n0 = tile_n * BN;
+    const int total_tiles = a.tiles_m * a.tiles_n;
+    int m0 = 0, n0 = 0;
     const int batch = blockIdx.y;
     const half_t* __restrict__ A = a.A + (size_t)batch * a.sa;
     const half_t* __restrict__ B = a.B + (size_t)batch * a.sb;
@@ -260,22 +264,34 @@ __global__ void __launch_bounds__(WM* WN * 64) hgemm_f16_dlds_kernel(HgemmArgs a
     const int ld_slot = lane % CPR;
     const half_t* a_src[A_LOADS];
     const half_t* b_src[B_LOADS];
+    const int KT_all = K / BK;
+    const int kt_begin = (int)blockIdx.z * a.kt_per_split;
+    const int KT = (KT_all - kt_begin) < a.kt_per_split ? (KT_all - kt_begin) : a.kt_per_split;
+    // tile `b` of the launch: sets m0, n0 and the per-lane source pointers (at this split's first K tile)
+    auto setup_tile = [&](int b) {
+        int tile_m, tile_n;
+        tile_of_block(b, total_tiles, a.tiles_m, tile_m, tile_n);
+        m0 = tile_m * BM;
+        n0 = tile_n * BN;
 #pragma unroll
-    for (int j = 0; j < A_LOADS; ++j) {
-        const int r = (j * NW + wave) * RPW + ld_row_in_group;  // tile row
-        const int c = ld_slot ^ ((r / RPL) % CPR);              // chunk of that row this lane fetches
-        int gr = m0 + r;
-        gr = gr < M ? gr : M - 1;
-        a_src[j] = A + (size_t)gr * K + c * 8;
-    }
+        for (int j = 0; j < A_LOADS; ++j) {
+            const int r = (j * NW + wave) * RPW + ld_row_in_group;  // tile row
+            const int c = ld_slot ^ ((r / RPL) % CPR);              // chunk of that row this lane fetches
+            int gr = m0 + r;
+            gr = gr < M ? gr : M - 1;
+            a_src[j] = A + (size_t)gr * K + c * 8 + (size_t)kt_begin * BK;
+        }
 #pragma unroll
-    for (int j = 0; j < B_LOADS; ++j) {
-        const int r = (j * NW + wave) * RPW + ld_row_in_group;
-        const int c = ld_slot ^ ((r / RPL) % CPR);
-        int gr = n0 + r;
-        gr = gr < N ? gr : N - 1;
-        b_src[j] = B + (size_t)gr * K + c * 8;
-    }
+        for (int j = 0; j < B_LOADS; ++j) {
+            const int r = (j * NW + wave) * RPW + ld_row_in_group;
+            const int c = ld_slot ^ ((r / RPL) % CPR);
+            int gr = n0 + r;
+            gr = gr < N ? gr : N - 1;
+            b_src[j] = B + (size_t)gr * K + c * 8 + (size_t)kt_begin * BK;
+        }
+    };
+    int vb = blockIdx.x;
+    setup_tile(vb);
     auto a_off = [&](int kt) { return (kt % STAGES) * STAGE_BYTES; };
     auto b_off = [&](int kt) { return (kt % STAGES) * STAGE_BYTES + A_BYTES; };
     auto issue_a = [&](int kt) {
@@ -311,20 +327,6 @@ __global__ void __launch_bounds__(WM* WN * 64) hgemm_f16_dlds_kernel(HgemmArgs a
     const int b_base = wn * TN * RB;
 
     float16_t acc[MT][NT];
-#pragma unroll
-    for (int i = 0; i < MT; ++i)
-#pragma unroll
-        for (int j = 0; j < NT; ++j)
-#pragma unroll
-            for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
-
-    const int KT_all = K / BK;
-    const int kt_begin = (int)blockIdx.z * a.kt_per_split;
-    const int KT = (KT_all - kt_begin) < a.kt_per_split ? (KT_all - kt_begin) : a.kt_per_split;
-#pragma unroll
-    for (int j = 0; j < A_LOADS; ++j) a_src[j] += (size_t)kt_begin * BK;
-#pragma unroll
-    for (int j = 0; j < B_LOADS; ++j) b_src[j] += (size_t)kt_begin * BK;
 #pragma unroll
     for (int s = 0; s < STAGES - 1; ++s)
         if (s < KT) { issue_a(s); issue_b(s); }
@@ -362,6 +364,14 @@ __global__ void __launch_bounds__(WM* WN * 64) hgemm_f16_dlds_kernel(HgemmArgs a
                 // registers, four CONSECUTIVE columns, which is what a vector store wants.
                 acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(bf[j], af[i], acc[i][j], 0, 0, 0);
     };
+
+  for (;;) {  // tiles of this workgroup (one, unless PERSIST)
+#pragma unroll
+    for (int i = 0; i < MT; ++i)
+#pragma unroll
+        for (int j = 0; j < NT; ++j)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
 
     if constexpr (MODE == 1) {
         // Fragments are double buffered in registers: the ds_reads of K step s+1 (or of the
@@ -437,6 +447,24 @@ __global__ void __launch_bounds__(WM* WN * 64) hgemm_f16_dlds_kernel(HgemmArgs a
     const int e_row = lane & 31;
     const int e_col = (lane >> 5) * 4;
     const int row_base = m0 + wm * TM, col_base = n0 + wn * TN;
+    constexpr int RS = TN * 2 + 16;          // bytes per staged row of the fp16 epilogue
+    const bool staged = !partial && (N % 8) == 0 && (reinterpret_cast<uintptr_t>(C) & 15u) == 0;
+    const int next_vb = vb + (int)gridDim.x;
+    const bool has_next_tile = PERSIST && next_vb < total_tiles;
+    if (staged || has_next_tile) {
+        // all wavefronts are done with the operand tiles before anyone overwrites them
+        asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    }
+    int stage_area = 0;
+    if constexpr (PERSIST) {
+        static_assert(!PERSIST || NW * 32 * RS <= STAGE_BYTES, "C staging must fit the second stage");
+        if (has_next_tile) {
+            // first K tile of the next C tile goes to stage 0 while this tile's C leaves through stage 1
+            setup_tile(next_vb);
+            if (KT > 0) { issue_a(0); issue_b(0); }
+            stage_area = STAGE_BYTES;
+        }
+    }
     if (partial) {
         // split-K: fp32 partial sums, four consecutive columns (16 bytes) per store where the row allows it
         const bool vec = (N % 4) == 0;
@@ -460,20 +488,15 @@ __global__ void __launch_bounds__(WM* WN * 64) hgemm_f16_dlds_kernel(HgemmArgs a
                     }
                 }
         }
-        return;
-    }
-    if ((N % 8) == 0 && (reinterpret_cast<uintptr_t>(C) & 15u) == 0) {
+    } else if (staged) {
         // fp16 output through LDS: every wavefront turns 32 x TN blocks of its accumulators into row-major
         // halves in a private LDS region (8-byte writes), reads them back 16 bytes per lane and stores
         // whole 16-byte pieces of C rows (TN = 64: full 128-byte lines).  Rows are padded by 16 bytes so
         // that the 32 rows of one write land in different banks.
-        constexpr int RS = TN * 2 + 16;          // bytes per staged row
         constexpr int CH = TN / 8;               // 16-byte chunks per row
         constexpr int RPR = 64 / CH;             // rows per wavefront-wide read
         static_assert(NW * 32 * RS <= STAGES * STAGE_BYTES, "staging area must fit the ring");
-        // all wavefronts are done with the operand tiles before anyone overwrites them
-        asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
-        unsigned char* region = smem_raw + wave * (32 * RS);
+        unsigned char* region = smem_raw + stage_area + wave * (32 * RS);
 #pragma unroll
         for (int i = 0; i < MT; ++i) {
 #pragma unroll
@@ -492,20 +515,23 @@ __global__ void __launch_bounds__(WM* WN * 64) hgemm_f16_dlds_kernel(HgemmArgs a
                 if (row < M && col < N) *reinterpret_cast<half8_t*>(C + (size_t)row * N + col) = v;
             }
         }
-        return;
+    } else {
+#pragma unroll
+        for (int i = 0; i < MT; ++i) {
+            const int row = row_base + i * 32 + e_row;
+            if (row >= M) continue;
+#pragma unroll
+            for (int j = 0; j < NT; ++j)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) {
+                    const int col = col_base + j * 32 + (e / 4) * 8 + e_col + (e % 4);
+                    if (col < N) C[(size_t)row * N + col] = (half_t)acc[i][j][e];
+                }
+        }
     }
-#pragma unroll
-    for (int i = 0; i < MT; ++i) {
-        const int row = row_base + i * 32 + e_row;
-        if (row >= M) continue;
-#pragma unroll
-        for (int j = 0; j < NT; ++j)
-#pragma unroll
-            for (int e = 0; e < 16; ++e) {
-                const int col = col_base + j * 32 + (e / 4) * 8 + e_col + (e % 4);
-                if (col < N) C[(size_t)row * N + col] = (half_t)acc[i][j][e];
-            }
-    }
+    if (!has_next_tile) break;
+    vb = next_vb;
+  }
 }
 
 // out[i] = half(sum over splits, in split order, of partial[s][i]): second pass of split-K.
@@ -775,7 +801,13 @@ int launch_hgemm(const void* A, const void* B, void* C, size_t M, size_t N, size
             if (rc != TL_OK) return rc;
         }
     }
-    hipLaunchKernelGGL(v.kernel, dim3((unsigned)nblocks, (unsigned)batch, (unsigned)splits), dim3(v.threads), lds, st, a);
+    // two-stage pipelined kernels are persistent: one workgroup per resident slot walks several tiles
+    size_t grid_x = nblocks;
+    if (v.stages == 2 && v.name[0] == 'p') {
+        const size_t resident = (size_t)device_info().cu_count * ((160 * 1024) / lds > 0 ? (160 * 1024) / lds : 1);
+        if (grid_x > resident) grid_x = resident;
+    }
+    hipLaunchKernelGGL(v.kernel, dim3((unsigned)grid_x, (unsigned)batch, (unsigned)splits), dim3(v.threads), lds, st, a);
     TL_CHECK_LAUNCH(v.name);
     if (splits > 1) {
         const size_t n = M * N;
