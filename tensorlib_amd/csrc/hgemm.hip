@@ -693,13 +693,14 @@ static int hgemm_variant_index(const char* name) {
 // round of at least 0.6 x CUs workgroups, with a deep (3-4 stage) ring; if even 128x64 tiles are too few,
 // K is split until the chip is full (see launch_hgemm).
 // More rows: the tile shape with the cheapest schedule.  One round of 256x256 tiles on every CU costs R; a
-// round of 128x256 tiles (one workgroup per CU) or of 128x128 tiles (two per CU) does half the work in
-// 0.57 R (0.63 R), so the big tile wins unless its last round is mostly empty; a partly filled round of a
-// fraction f of the CUs costs about (0.65 + 0.3 f) of a full one (fewer busy CUs clock higher).  Splitting K
-// or peeling the last round off into a second K-split launch lost to this on every shape tried.
+// round of 128x256 tiles (one workgroup per CU, three-stage ring: with B streamed from HBM a 0.6 us tile step
+// is shorter than the memory latency two stages can hide) does half the work in 0.61 R, a round of 128x128
+// tiles (two per CU) in 0.66 R, so the big tile wins unless its last round is mostly empty; a partly filled
+// round of a fraction f of the CUs costs about (0.65 + 0.3 f) of a full one (fewer busy CUs clock higher).
+// Splitting K or peeling the last round off into a second K-split launch lost to this on every shape tried.
 static int pick_variant(size_t M, size_t N, size_t K, int cus) {
     static const int v_big = hgemm_variant_index("p256x256x64w2x4s2");
-    static const int v_mid = hgemm_variant_index("p128x256x64w2x4s2");
+    static const int v_mid = hgemm_variant_index("p128x256x64w2x4s3");
     static const int v_small = hgemm_variant_index("p128x128x64w2x4s2");
     static const int v_few_256x128 = hgemm_variant_index("p256x128x64w2x4s3");
     static const int v_few_128x128 = hgemm_variant_index("p128x128x64w2x4s4");
@@ -713,13 +714,15 @@ static int pick_variant(size_t M, size_t N, size_t K, int cus) {
         if (tiles(128, 128) >= enough || (K >= 8192 && tiles(128, 128) * 2 >= enough)) return v_few_128x128;
         return v_few_128x64;
     }
+    // a problem that leaves half the CUs without a 128x256 tile spreads wider as 128x128 tiles
+    if (tiles(128, 256) * 2 <= (size_t)cus) return v_few_128x128;
     auto cost = [&](size_t t, size_t slots, double round_cost) {
         const size_t full = t / slots, rem = t % slots;
         return round_cost * ((double)full + (rem ? 0.65 + 0.3 * (double)rem / (double)slots : 0.0));
     };
     const double c_big = cost(tiles(256, 256), (size_t)cus, 1.0);
-    const double c_mid = cost(tiles(128, 256), (size_t)cus, 0.565);
-    const double c_small = cost(tiles(128, 128), (size_t)cus * 2, 0.63);
+    const double c_mid = cost(tiles(128, 256), (size_t)cus, 0.613);
+    const double c_small = cost(tiles(128, 128), (size_t)cus * 2, 0.66);
     int best = v_big;
     double c = c_big;
     if (c_mid < c * 0.97) { best = v_mid; c = c_mid; }
