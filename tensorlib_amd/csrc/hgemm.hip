@@ -231,11 +231,12 @@ __global__ void __launch_bounds__(WM* WN * 64) hgemm_f16_dlds_kernel(HgemmArgs a
     static_assert(BK == 32 || BK == 64, "BK must be 32 or 64");
     static_assert(BM % (RPW * NW) == 0 && BN % (RPW * NW) == 0, "tile rows must split over the wavefronts");
     static_assert(STAGES >= 2 && STAGES <= 5 && LPW * (STAGES - 2) < 64, "vmcnt is a 6-bit counter");
-    // Two-stage pipelined variants are persistent: a workgroup walks tiles blockIdx.x, + gridDim.x, ... and
-    // requests the first K tile of its next C tile before it stores the current one, so the C stores and
-    // the cold start of the next tile overlap.  (vmcnt counts loads and stores together on this ISA, which
-    // is fine for two stages: every tile barrier waits for vmcnt(0) anyway.)
-    constexpr bool PERSIST = (STAGES == 2 && MODE == 1);
+    // Pipelined variants with two or three stages are persistent: a workgroup walks tiles blockIdx.x,
+    // + gridDim.x, ... and requests the first STAGES-1 K tiles of its next C tile before it stores the current
+    // one (staged through the last stage's LDS), so the C stores and the cold start of the next tile overlap.
+    // vmcnt counts loads and stores together on this ISA, so the stores are drained (vmcnt(0)) before the
+    // next tile's loop resumes waiting with exact load counts.
+    constexpr bool PERSIST = (STAGES <= 3 && MODE == 1);
 
     extern __shared__ __attribute__((aligned(1024))) unsigned char smem_raw[];
     typedef __attribute__((address_space(3))) unsigned char lds_byte_t;
@@ -457,12 +458,15 @@ __global__ void __launch_bounds__(WM* WN * 64) hgemm_f16_dlds_kernel(HgemmArgs a
     }
     int stage_area = 0;
     if constexpr (PERSIST) {
-        static_assert(!PERSIST || NW * 32 * RS <= STAGE_BYTES, "C staging must fit the second stage");
+        static_assert(!PERSIST || NW * 32 * RS <= STAGE_BYTES, "C staging must fit the last stage");
         if (has_next_tile) {
-            // first K tile of the next C tile goes to stage 0 while this tile's C leaves through stage 1
+            // the first K tiles of the next C tile go to stages 0 .. STAGES-2 while this tile's C leaves
+            // through the last stage
             setup_tile(next_vb);
-            if (KT > 0) { issue_a(0); issue_b(0); }
-            stage_area = STAGE_BYTES;
+#pragma unroll
+            for (int st = 0; st < STAGES - 1; ++st)
+                if (st < KT) { issue_a(st); issue_b(st); }
+            stage_area = (STAGES - 1) * STAGE_BYTES;
         }
     }
     if (partial) {
@@ -530,6 +534,7 @@ __global__ void __launch_bounds__(WM* WN * 64) hgemm_f16_dlds_kernel(HgemmArgs a
         }
     }
     if (!has_next_tile) break;
+    if constexpr (STAGES > 2) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     vb = next_vb;
   }
 }
@@ -804,9 +809,9 @@ int launch_hgemm(const void* A, const void* B, void* C, size_t M, size_t N, size
             if (rc != TL_OK) return rc;
         }
     }
-    // two-stage pipelined kernels are persistent: one workgroup per resident slot walks several tiles
+    // pipelined kernels with up to three stages are persistent: one workgroup per resident slot walks several tiles
     size_t grid_x = nblocks;
-    if (v.stages == 2 && v.name[0] == 'p') {
+    if (v.stages <= 3 && v.name[0] == 'p') {
         const size_t resident = (size_t)device_info().cu_count * ((160 * 1024) / lds > 0 ? (160 * 1024) / lds : 1);
         if (grid_x > resident) grid_x = resident;
     }
