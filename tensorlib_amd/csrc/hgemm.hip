@@ -10,11 +10,12 @@
 // half-wavefronts supply k 0..7 and 8..15.  So a 16-byte global load, a 16-byte LDS write
 // and a 16-byte LDS read move an operand fragment without any shuffling.
 //
-// Tiling: a workgroup of WM x WN wavefronts owns a BM x BN tile of C and walks K in steps
-// of BK.  Tiles of A and B are staged in LDS rows of BK+8 halves (the 16-byte pad makes the
-// 32 rows a ds_read_b128 touches fall in distinct bank groups), double buffered: while the
-// MFMAs of step k run out of one buffer, the global loads of step k+1 are in flight in
-// registers and are written to the other buffer before the single barrier of the step.
+// Two kernels share that layout.  hgemm_f16_dlds_kernel (K % 64 == 0, the prefill shapes) moves tiles
+// global -> LDS with global_load_lds_dwordx4 through a ring of stages, swizzles the chunk order instead of
+// padding rows, pipelines fragment reads under the MFMAs of the previous K step and, for rings of two or
+// three stages, is persistent over C tiles.  hgemm_f16_mfma_kernel (any K % 8 == 0) stages tiles through
+// registers into LDS rows of BK+8 halves (the 16-byte pad makes the 32 rows a ds_read_b128 touches fall
+// in distinct bank groups) and zero-fills the K tail.  gemm_generic_kernel covers everything else.
 #include <cstring>
 #include <mutex>
 #include <type_traits>
@@ -608,48 +609,27 @@ struct HgemmVariant {
 
 static const HgemmVariant g_variants[] = {
     {"auto", 0, 0, 0, 0, 0, nullptr},
+    // register-staged kernel: serves K % 64 != 0 (index 1 is the fallback of launch_hgemm)
     TL_HGEMM_VARIANT(128, 128, 64, 2, 2),  // 1
-    TL_HGEMM_VARIANT(256, 128, 64, 2, 2),  // 2
-    TL_HGEMM_VARIANT(128, 256, 64, 2, 2),  // 3
-    TL_HGEMM_VARIANT(256, 256, 64, 2, 2),  // 4
-    TL_HGEMM_VARIANT(64, 64, 64, 2, 2),    // 5
-    TL_HGEMM_VARIANT(256, 256, 32, 2, 2),  // 6
-    TL_HGEMM_VARIANT(128, 128, 32, 2, 2),  // 7
-    TL_HGEMM_VARIANT(64, 128, 64, 2, 2),   // 8
-    TL_HGEMM_VARIANT(256, 256, 64, 2, 4),  // 9   8 wavefronts, 128x64 each
-    TL_HGEMM_VARIANT(256, 256, 64, 4, 2),  // 10  8 wavefronts, 64x128 each
-    TL_HGEMM_VARIANT(256, 256, 32, 2, 4),  // 11
-    TL_HGEMM_VARIANT(256, 128, 64, 2, 4),  // 12  128x32 each
-    TL_HGEMM_VARIANT(256, 128, 64, 4, 2),  // 13  64x64 each
-    TL_HGEMM_VARIANT(128, 256, 64, 2, 4),  // 14  64x64 each
-    TL_HGEMM_VARIANT(128, 128, 64, 2, 4),  // 15  64x32 each
-    TL_HGEMM_DLDS(256, 256, 64, 2, 4, 2),  // 16
-    TL_HGEMM_DLDS(256, 256, 64, 2, 2, 2),  // 17
-    TL_HGEMM_DLDS(256, 256, 32, 2, 4, 4),  // 18
-    TL_HGEMM_DLDS(256, 256, 32, 2, 4, 3),  // 19
-    TL_HGEMM_DLDS(256, 256, 32, 2, 2, 4),  // 20
-    TL_HGEMM_DLDS(256, 128, 64, 2, 4, 3),  // 21
-    TL_HGEMM_DLDS(256, 128, 64, 2, 2, 3),  // 22
-    TL_HGEMM_DLDS(128, 256, 64, 2, 4, 3),  // 23
-    TL_HGEMM_DLDS(128, 128, 64, 2, 2, 4),  // 24
-    TL_HGEMM_DLDS(128, 128, 64, 2, 2, 2),  // 25
-    TL_HGEMM_DLDS(256, 128, 32, 2, 4, 4),  // 26
-    TL_HGEMM_DLDS(128, 128, 32, 2, 2, 4),  // 27
-    TL_HGEMM_PIPE(256, 256, 64, 2, 4, 2),  // 28
-    TL_HGEMM_PIPE(256, 256, 64, 2, 2, 2),  // 29
-    TL_HGEMM_PIPE(256, 128, 64, 2, 4, 2),  // 30
-    TL_HGEMM_PIPE(128, 256, 64, 2, 4, 2),  // 31
-    TL_HGEMM_PIPE(128, 256, 64, 2, 4, 3),  // 32
-    TL_HGEMM_PIPE(128, 128, 64, 2, 2, 2),  // 33
-    TL_HGEMM_PIPE(256, 128, 64, 2, 2, 2),  // 34
-    TL_HGEMM_PIPE(128, 256, 64, 2, 2, 2),  // 35
-    TL_HGEMM_PIPE(128, 128, 64, 2, 4, 2),  // 36
-    TL_HGEMM_PIPE(256, 256, 32, 2, 4, 4),  // 37
-    TL_HGEMM_PIPE(128, 64, 64, 2, 2, 4),   // 38  few rows: narrow B tiles, deep ring
-    TL_HGEMM_PIPE(128, 64, 64, 4, 1, 4),   // 39
-    TL_HGEMM_PIPE(128, 128, 64, 2, 4, 4),  // 40
-    TL_HGEMM_PIPE(256, 128, 64, 2, 4, 3),  // 41
+    TL_HGEMM_VARIANT(256, 256, 64, 2, 4),  // 2
+    TL_HGEMM_VARIANT(64, 64, 64, 2, 2),    // 3
+    // direct-to-LDS ring, fragments read step by step (no register double buffering)
+    TL_HGEMM_DLDS(256, 256, 64, 2, 4, 2),  // 4
+    TL_HGEMM_DLDS(128, 128, 64, 2, 2, 4),  // 5
+    TL_HGEMM_DLDS(256, 256, 32, 2, 4, 4),  // 6   BK = 32: half cache lines per row, measured slower
+    // direct-to-LDS ring, pipelined (dispatch picks among these)
+    TL_HGEMM_PIPE(256, 256, 64, 2, 4, 2),  // 7   8 wavefronts of 128x64
+    TL_HGEMM_PIPE(256, 256, 64, 2, 2, 2),  // 8   4 wavefronts of 128x128
+    TL_HGEMM_PIPE(128, 256, 64, 2, 4, 2),  // 9
+    TL_HGEMM_PIPE(128, 256, 64, 2, 4, 3),  // 10
+    TL_HGEMM_PIPE(256, 128, 64, 2, 4, 2),  // 11
+    TL_HGEMM_PIPE(256, 128, 64, 2, 4, 3),  // 12
+    TL_HGEMM_PIPE(128, 128, 64, 2, 4, 2),  // 13
+    TL_HGEMM_PIPE(128, 128, 64, 2, 4, 4),  // 14
+    TL_HGEMM_PIPE(128, 64, 64, 2, 2, 4),   // 15  few rows: narrow B tiles, deep ring
+    TL_HGEMM_PIPE(128, 64, 64, 4, 1, 4),   // 16
 };
+
 static constexpr int kNumVariants = sizeof(g_variants) / sizeof(g_variants[0]);
 static int g_forced_variant = 0;
 static bool g_attr_set[kNumVariants] = {false};
