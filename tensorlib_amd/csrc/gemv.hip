@@ -422,42 +422,28 @@ struct GemvVariant {
 
 static const GemvVariant g_variants[] = {
     {"auto", 0, 0, 0, 0, 0, nullptr},
-    TL_LOOP(4, 2, 8, 1, false),   // 1
-    TL_LOOP(4, 2, 8, 1, true),    // 2
-    TL_LOOP(4, 4, 8, 1, true),    // 3
-    TL_LOOP(4, 2, 4, 2, true),    // 4
-    TL_LOOP(4, 2, 6, 4, false),   // 5
-    TL_LOOP(4, 2, 6, 4, true),    // 6
-    TL_LOOP(8, 2, 6, 4, true),    // 7
-    TL_LOOP(4, 2, 2, 4, true),    // 8
-    // K = 4096 candidates (512 chunks per row)
-    TL_STREAM2(4, 2, 2, 4),       // 9, 10
-    TL_STREAM2(4, 4, 2, 4),       // 11, 12
-    TL_STREAM2(4, 8, 2, 4),       // 13, 14
-    TL_STREAM2(4, 2, 4, 2),       // 15, 16
-    TL_STREAM2(4, 4, 4, 2),       // 17, 18
-    TL_STREAM2(4, 1, 8, 1),       // 19, 20
-    TL_STREAM2(4, 2, 8, 1),       // 21, 22
-    TL_STREAM2(8, 2, 1, 8),       // 23, 24
-    TL_STREAM2(8, 4, 1, 8),       // 25, 26
-    TL_STREAM2(8, 2, 2, 4),       // 27, 28
-    TL_STREAM2(8, 4, 2, 4),       // 29, 30
-    // K = 11008 candidates (1376 chunks per row)
-    TL_STREAM2(4, 2, 6, 4),       // 31, 32
-    TL_STREAM2(4, 4, 6, 4),       // 33, 34
-    TL_STREAM2(8, 2, 3, 8),       // 35, 36
-    TL_STREAM2(8, 4, 3, 8),       // 37, 38
-    TL_STREAM2(4, 1, 11, 2),      // 39, 40
-    TL_STREAM2(4, 2, 11, 2),      // 41, 42
-    TL_STREAM2(8, 2, 6, 4),       // 43, 44
-    TL_STREAM2(8, 1, 6, 4),       // 45, 46
-    TL_STREAM2(4, 1, 6, 4),       // 47, 48
-    TL_STREAM2(4, 1, 2, 4),       // 49, 50
-    TL_STREAM(4, 2, 2, 4, 2),     // 51  silu*mul prologue, K <= 4096
-    TL_STREAM(8, 2, 3, 8, 2),     // 52  silu*mul prologue, K <= 12288
-    TL_STREAM(4, 2, 2, 4, 3),     // 53  add + RMSNorm prologue, K <= 4096
-    TL_STREAM(8, 2, 3, 8, 3),     // 54  add + RMSNorm prologue, K <= 12288
+    // looping kernel, x staged in LDS (any K)
+    TL_LOOP(4, 2, 8, 1, true),    // 1
+    TL_LOOP(4, 2, 6, 4, false),   // 2
+    TL_LOOP(4, 2, 6, 4, true),    // 3   K > 12288
+    TL_LOOP(8, 2, 6, 4, true),    // 4
+    // K = 4096 (512 chunks per row): x in LDS (x0) against x in registers (x1)
+    TL_STREAM2(4, 2, 2, 4),       // 5, 6    6 = dispatch for K <= 4096
+    TL_STREAM2(4, 4, 2, 4),       // 7, 8
+    TL_STREAM2(4, 2, 4, 2),       // 9, 10
+    TL_STREAM2(4, 2, 8, 1),       // 11, 12
+    TL_STREAM2(8, 2, 2, 4),       // 13, 14
+    // K = 11008 (1376 chunks per row)
+    TL_STREAM2(8, 2, 3, 8),       // 15, 16  16 = dispatch for K <= 12288
+    TL_STREAM2(4, 2, 6, 4),       // 17, 18
+    TL_STREAM2(8, 2, 6, 4),       // 19, 20
+    TL_STREAM2(4, 2, 11, 2),      // 21, 22
+    TL_STREAM(4, 2, 2, 4, 2),     // 23  silu*mul prologue, K <= 4096
+    TL_STREAM(8, 2, 3, 8, 2),     // 24  silu*mul prologue, K <= 12288
+    TL_STREAM(4, 2, 2, 4, 3),     // 25  add + RMSNorm prologue, K <= 4096
+    TL_STREAM(8, 2, 3, 8, 3),     // 26  add + RMSNorm prologue, K <= 12288
 };
+
 static constexpr int kNumVariants = sizeof(g_variants) / sizeof(g_variants[0]);
 static int g_forced_variant = 0;
 static int g_grid_waves_per_cu = 0;  // 0 = automatic
