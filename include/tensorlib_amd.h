@@ -229,6 +229,20 @@ int tl_prefill_rope_qkv_f16(void* q_out, const void* q, const void* k, const voi
                             void* cache_k, void* cache_v, const void* rope_table, int start_pos, int n_tokens,
                             int n_heads, int head_dim);
 
+/* vT[h][d][t] = cache_v[t][h][d] for t < T and 0 for T <= t < ldv (ldv % 8 == 0): the transposed value operand
+ * of tl_prefill_attention_f16; the reference builds the same tensor with transpose + contiguous
+ * (model/llama2_7b/src/Transformer.cpp:66-80). */
+int tl_gather_vt_f16(void* vT, const void* cache_v, int T, int ldv, int n_heads, int head_dim);
+
+/* Causal attention of n_tokens new tokens over cache positions [0, start_pos + n_tokens) in one launch:
+ * scores, ScalarDiv by half(sqrt(head_dim)), mask, softmax and the product with the values
+ * (Attention::forward, model/llama2_7b/src/Transformer.cpp:92-109) without a score matrix in memory.
+ * q: [n_heads, n_tokens, head_dim] (rotated, as tl_prefill_rope_qkv_f16 writes it); cache_k: [.., n_heads,
+ * head_dim]; vT from tl_gather_vt_f16 with ldv >= the context rounded up to 32; out: [n_tokens, n_heads,
+ * head_dim].  head_dim 64 or 128. */
+int tl_prefill_attention_f16(void* out, const void* q, const void* cache_k, const void* vT, int ldv, int start_pos,
+                             int n_tokens, int n_heads, int head_dim);
+
 /* In place on scores [n_heads, seqlen, start_pos + seqlen]: ScalarDiv by `divisor` (fp16 bits), the causal
  * mask add and softmax(3) of Attention::forward (model/llama2_7b/src/Transformer.cpp:94-105) in one launch;
  * the quotient is rounded to fp16 before the softmax, as the separate kernels store it. */

@@ -82,6 +82,8 @@ _PROTOS = {
     "tl_prefill_rope_qkv_f16": (_i, [_vp, _vp, _vp, _vp, _sz, _vp, _vp, _vp, _i, _i, _i, _i]),
     "tl_scaled_causal_softmax_f16": (_i, [_vp, _u16, _i, _i, _i]),
     "tl_silu_mul_rows_f16": (_i, [_vp, _vp, _sz, _sz]),
+    "tl_gather_vt_f16": (_i, [_vp, _vp, _i, _i, _i, _i]),
+    "tl_prefill_attention_f16": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i]),
     "tl_gemv_add_rms_norm_f16": (_i, [_vp, _vp, _vp, _f, _vp, _vp, _vp, _sz, _sz]),
     "tl_decode_attention_rope_f16": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i]),
     "tl_rope_table_f16": (_i, [_vp, _i, _i]),

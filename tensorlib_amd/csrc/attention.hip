@@ -278,6 +278,152 @@ prefill_rope_qkv_kernel(half_t* q_out, const half_t* q, const half_t* k, const h
     *reinterpret_cast<half2_t*>(cache_v + c_off) = vv;
 }
 
+// vT[h][d][t] = cache_v[t][h][d] for t < T, zero for T <= t < ldv: the value operand of the prefill attention,
+// rows of `ldv` elements (a multiple of 8, so that groups of four positions can be read with 8-byte loads).
+__global__ void __launch_bounds__(256)
+gather_vt_kernel(half_t* vT, const half_t* cache_v, int T, int ldv, int n_heads, int head_dim) {
+    __shared__ half_t tile[64][65];
+    const int h = blockIdx.z;
+    const int t0 = blockIdx.x * 64, d0 = blockIdx.y * 64;
+    const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;  // 64 x 4
+    for (int r = ty; r < 64; r += 4) {
+        const int t = t0 + r, d = d0 + tx;
+        tile[r][tx] = (t < T && d < head_dim) ? cache_v[((size_t)t * n_heads + h) * head_dim + d] : (half_t)0.f;
+    }
+    __syncthreads();
+    for (int r = ty; r < 64; r += 4) {
+        const int d = d0 + r, t = t0 + tx;
+        if (d < head_dim && t < ldv) vT[((size_t)h * head_dim + d) * ldv + t] = tile[tx][r];
+    }
+}
+
+// Causal attention of n_tokens new tokens against cache positions [0, start_pos + n_tokens): one wavefront per
+// (head, 32 query rows), no LDS, no score matrix in memory.  Per block of 32 keys:
+//   S^T[key][q] = sum_d K[key][d] Q[q][d]        8 MFMAs, A = K rows straight from the cache, B = Q (registers)
+//   lane l then holds 16 keys of ONE query row (l % 32): the online-softmax row reductions are in-lane plus
+//   one exchange with lane l ^ 32; scores are rounded like the reference chain (fp16 score, fp16 quotient by
+//   half(sqrt(head_dim)), -inf above the diagonal);
+//   O^T[d][q] += sum_key vT[d][key] P^T[key][q]   A = vT with the key order the accumulator layout dictates
+//   (lane half h of MFMA step s owns keys 16s+4h+{0..3} and 16s+8+4h+{0..3}: two 8-byte loads), B = P^T taken
+//   from the score accumulators of the same lane without any shuffle.
+// q: [n_heads, n_tokens, D] (rotated), out: [n_tokens, n_heads, D].
+// One wavefront per workgroup: the kernel is bound by memory latency, so the (head, query block) units are
+// spread over as many CUs as possible, the K rows of the next key block and the value fragments of the
+// current one are requested before the score MFMAs of the current block start.
+template <int D>
+__global__ void __launch_bounds__(64)
+prefill_attention_kernel(half_t* out, const half_t* q, const half_t* cache_k, const half_t* vT, int ldv, int start_pos,
+                         int n_tokens, int n_heads, half_t divisor) {
+    constexpr int KS = D / 16;    // MFMA steps over head_dim for Q.K
+    constexpr int DB = D / 32;    // 32-row blocks of O^T
+    const int lane = threadIdx.x & 63;
+    const int h = blockIdx.y;
+    const int qb = blockIdx.x;                      // block of 32 query rows
+    const int q0 = qb * 32;
+    if (q0 >= n_tokens) return;
+    const int T = start_pos + n_tokens;
+    const int lr = lane & 31, lh = lane >> 5;
+    const int my_q = q0 + lr;                       // the query row this lane owns in S^T / O^T
+    const int my_q_c = my_q < n_tokens ? my_q : n_tokens - 1;
+    const int limit = start_pos + my_q;             // last visible key
+    const float dv = (float)divisor;
+
+    half8_t qf[KS];
+    const half_t* qrow = q + ((size_t)h * n_tokens + my_q_c) * D + lh * 8;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) qf[ks] = *reinterpret_cast<const half8_t*>(qrow + ks * 16);
+
+    float16_t o[DB];
+#pragma unroll
+    for (int b = 0; b < DB; ++b)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) o[b][e] = 0.f;
+    float m = -INFINITY, l = 0.f;
+
+    const int last_key = start_pos + (q0 + 31 < n_tokens ? q0 + 31 : n_tokens - 1);  // of the whole wavefront
+    const size_t krow_stride = (size_t)n_heads * D;
+    auto load_k = [&](half8_t (&dst)[KS], int t0) {
+        int key = t0 + lr;
+        key = key < T ? key : T - 1;
+        const half_t* krow = cache_k + (size_t)key * krow_stride + (size_t)h * D + lh * 8;
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) dst[ks] = *reinterpret_cast<const half8_t*>(krow + ks * 16);
+    };
+    half8_t kf[KS], kn[KS];
+    load_k(kf, 0);
+    for (int t0 = 0; t0 <= last_key; t0 += 32) {
+        // requests for the next block's K rows and this block's value fragments go out first
+        if (t0 + 32 <= last_key) load_k(kn, t0 + 32);
+        half4_t vraw[DB][2][2];
+#pragma unroll
+        for (int b = 0; b < DB; ++b) {
+            const half_t* vrow = vT + ((size_t)h * D + b * 32 + lr) * ldv + t0 + 4 * lh;
+#pragma unroll
+            for (int st = 0; st < 2; ++st) {
+                vraw[b][st][0] = *reinterpret_cast<const half4_t*>(vrow + 16 * st);
+                vraw[b][st][1] = *reinterpret_cast<const half4_t*>(vrow + 16 * st + 8);
+            }
+        }
+        // ---- S^T block ----
+        float16_t sacc;
+#pragma unroll
+        for (int e = 0; e < 16; ++e) sacc[e] = 0.f;
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) sacc = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf[ks], qf[ks], sacc, 0, 0, 0);
+        // sacc[4g + r] = score of key t0 + 8g + 4*lh + r against query my_q
+        float sv[16];
+        float bm = -INFINITY;
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+            const int kk = t0 + 8 * (e / 4) + 4 * lh + (e % 4);
+            const half_t s16 = (half_t)sacc[e];
+            const float t = (float)(half_t)((float)s16 / dv);
+            sv[e] = kk <= limit ? t : -INFINITY;
+            bm = fmaxf(bm, sv[e]);
+        }
+        bm = fmaxf(bm, __shfl_xor(bm, 32, 64));
+        const float m_new = fmaxf(m, bm);
+        const float corr = (m == -INFINITY) ? 0.f : expf(m - m_new);
+        float bs = 0.f;
+        half8_t pf[2];
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+            const float pv = (m_new == -INFINITY) ? 0.f : expf(sv[e] - m_new);
+            const half_t p16 = (half_t)pv;
+            bs += (float)p16;
+            pf[e / 8][e % 8] = p16;       // step s = e / 8 holds g = 2s (slots 0..3) and g = 2s + 1 (slots 4..7)
+        }
+        bs += __shfl_xor(bs, 32, 64);
+        l = l * corr + bs;
+        m = m_new;
+        // ---- O^T += vT . P^T ----
+#pragma unroll
+        for (int b = 0; b < DB; ++b) {
+#pragma unroll
+            for (int e = 0; e < 16; ++e) o[b][e] *= corr;
+#pragma unroll
+            for (int st = 0; st < 2; ++st) {
+                const half4_t v0 = vraw[b][st][0], v1 = vraw[b][st][1];
+                const half8_t vf = {v0[0], v0[1], v0[2], v0[3], v1[0], v1[1], v1[2], v1[3]};
+                o[b] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf, pf[st], o[b], 0, 0, 0);
+            }
+        }
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) kf[ks] = kn[ks];
+    }
+    if (my_q >= n_tokens) return;
+    const float inv = 1.0f / l;
+    half_t* orow = out + ((size_t)my_q * n_heads + h) * D;
+#pragma unroll
+    for (int b = 0; b < DB; ++b)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            half4_t r = {(half_t)(o[b][4 * g] * inv), (half_t)(o[b][4 * g + 1] * inv), (half_t)(o[b][4 * g + 2] * inv),
+                         (half_t)(o[b][4 * g + 3] * inv)};
+            *reinterpret_cast<half4_t*>(orow + b * 32 + 8 * g + 4 * lh) = r;
+        }
+}
+
 // Decode-step glue after the fused q|k|v GEMV: rotate q in place, rotate k and write it to
 // cache_k[pos], copy v to cache_v[pos].  One thread per (even, odd) pair of the 3*dim vector.
 __global__ void __launch_bounds__(256)
@@ -508,6 +654,45 @@ int tl_prefill_rope_qkv_f16(void* q_out, const void* q, const void* k, const voi
                        (tl::half_t*)cache_k, (tl::half_t*)cache_v, (const tl::half_t*)rope_table, start_pos, n_tokens,
                        n_heads, head_dim);
     TL_CHECK_LAUNCH("prefill_rope_qkv_kernel");
+    return TL_OK;
+}
+
+int tl_gather_vt_f16(void* vT, const void* cache_v, int T, int ldv, int n_heads, int head_dim) {
+    TL_ENSURE_INIT();
+    TL_REQUIRE(vT && cache_v, "tl_gather_vt_f16: null pointer");
+    TL_REQUIRE(T >= 1 && ldv >= T && ldv % 8 == 0 && n_heads >= 1 && head_dim >= 1, "tl_gather_vt_f16: bad sizes");
+    TL_REQUIRE(n_heads <= 65535, "tl_gather_vt_f16: too many heads");
+    dim3 grid((unsigned)((ldv + 63) / 64), (unsigned)((head_dim + 63) / 64), (unsigned)n_heads);
+    hipLaunchKernelGGL(tl::gather_vt_kernel, grid, dim3(256), 0, tl::stream(), (tl::half_t*)vT, (const tl::half_t*)cache_v,
+                       T, ldv, n_heads, head_dim);
+    TL_CHECK_LAUNCH("gather_vt_kernel");
+    return TL_OK;
+}
+
+int tl_prefill_attention_f16(void* out, const void* q, const void* cache_k, const void* vT, int ldv, int start_pos,
+                             int n_tokens, int n_heads, int head_dim) {
+    TL_ENSURE_INIT();
+    TL_REQUIRE(out && q && cache_k && vT, "tl_prefill_attention_f16: null pointer");
+    TL_REQUIRE(start_pos >= 0 && n_tokens >= 1 && n_heads >= 1 && n_heads <= 65535, "tl_prefill_attention_f16: bad sizes");
+    TL_REQUIRE(head_dim == 64 || head_dim == 128, "tl_prefill_attention_f16: head_dim %d not supported (64 or 128)",
+               head_dim);
+    // the value reads run to the end of the last block of 32 keys
+    TL_REQUIRE(ldv % 8 == 0 && ldv >= ((start_pos + n_tokens + 31) / 32) * 32,
+               "tl_prefill_attention_f16: ldv=%d must be a multiple of 8 and cover the context rounded up to 32", ldv);
+    TL_REQUIRE(tl::aligned16(q) && tl::aligned16(cache_k) && tl::aligned16(vT) && tl::aligned16(out),
+               "tl_prefill_attention_f16: operands must be 16-byte aligned");
+    const float sq = sqrtf((float)head_dim);
+    const tl::half_t divisor = (tl::half_t)sq;  // the reference divides by half(sqrt(head_dim)) (Transformer.cpp:94)
+    dim3 grid((unsigned)((n_tokens + 31) / 32), (unsigned)n_heads);
+    if (head_dim == 64)
+        hipLaunchKernelGGL(tl::prefill_attention_kernel<64>, grid, dim3(64), 0, tl::stream(), (tl::half_t*)out,
+                           (const tl::half_t*)q, (const tl::half_t*)cache_k, (const tl::half_t*)vT, ldv, start_pos, n_tokens,
+                           n_heads, divisor);
+    else
+        hipLaunchKernelGGL(tl::prefill_attention_kernel<128>, grid, dim3(64), 0, tl::stream(), (tl::half_t*)out,
+                           (const tl::half_t*)q, (const tl::half_t*)cache_k, (const tl::half_t*)vT, ldv, start_pos, n_tokens,
+                           n_heads, divisor);
+    TL_CHECK_LAUNCH("prefill_attention_kernel");
     return TL_OK;
 }
 

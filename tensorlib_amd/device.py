@@ -389,6 +389,20 @@ class HipDevice:
         check(self.lib.tl_silu_mul_rows_f16(_ptr(out), _ptr(ab), rows, two_h // 2), "tl_silu_mul_rows_f16")
         return out
 
+    def prefill_attention(self, q: torch.Tensor, cache_k: torch.Tensor, cache_v: torch.Tensor, start_pos: int):
+        """q: [n_heads, S, head_dim] (rotated); caches [max_seq, n_heads, head_dim] holding positions
+        < start_pos + S.  Returns [S, n_heads, head_dim]."""
+        _req(q, name="q"), _req(cache_k, name="cache_k"), _req(cache_v, name="cache_v")
+        H, S, D = q.shape
+        T = start_pos + S
+        ldv = (T + 31) // 32 * 32
+        vT = self.empty(H, D, ldv)
+        check(self.lib.tl_gather_vt_f16(_ptr(vT), _ptr(cache_v), T, ldv, H, D), "tl_gather_vt_f16")
+        out = self.empty(S, H, D)
+        check(self.lib.tl_prefill_attention_f16(_ptr(out), _ptr(q), _ptr(cache_k), _ptr(vT), ldv, start_pos, S, H, D),
+              "tl_prefill_attention_f16")
+        return out
+
     # -- tuning hooks -------------------------------------------------------------------
     def set_gemv_variant(self, v: int) -> None:
         check(self.lib.tl_set_gemv_variant(v), "tl_set_gemv_variant")

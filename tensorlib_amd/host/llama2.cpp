@@ -263,9 +263,10 @@ struct tlm_model {
     }
 
     // Prefill of S > 1 tokens with the glue ops fused: one q|k|v GEMM and one w1|w3 GEMM when the weights
-    // are adjacent, RoPE + cache write + q transpose in one launch, ScalarDiv + mask + softmax in one launch,
-    // residual add + RMSNorm in one launch, SwiGLU gate in one launch.  14 launches per layer instead of 27;
-    // the matmuls are the same calls as in the reference chain.  Leaves rmsnorm(x) * final_norm in x_norm.
+    // are adjacent, RoPE + cache write + q transpose in one launch, the whole causal attention in one launch
+    // (head_dim 64/128; otherwise per-head matmuls with ScalarDiv + mask + softmax fused), residual add +
+    // RMSNorm in one launch, SwiGLU gate in one launch.  10 launches per layer instead of 27; the projections
+    // are the same matmul2d calls as in the reference chain.  Leaves rmsnorm(x) * final_norm in x_norm.
     void prefill_fused(int S, int start_pos) {
         const int T = start_pos + S, H = n_heads, D = head_dim;
         const size_t sd = (size_t)S * dim;
@@ -288,6 +289,14 @@ struct tlm_model {
             }
             ck(tl_prefill_rope_qkv_f16(xq_c.p, q, k, v, ld, cache_k[l].p, cache_v[l].p, rope_table.p, start_pos, S, H, D),
                "prefill_rope_qkv");
+            if (D == 64 || D == 128) {
+                // scores, scale, mask, softmax and the product with the values in one launch, keys read from the
+                // cache in place; only the values are transposed first                     Transformer.cpp:61-109
+                const int ldv = (T + 31) / 32 * 32;
+                ck(tl_gather_vt_f16(values_c.p, cache_v[l].p, T, ldv, H, D), "gather_vt");
+                ck(tl_prefill_attention_f16(o_c.p, xq_c.p, cache_k[l].p, values_c.p, ldv, start_pos, S, H, D),
+                   "prefill_attention");
+            } else {
             // keys -> [H,T,D], values -> [H,D,T] (what the per-head matmul2d calls consume)   Transformer.cpp:61-80
             cache_k[l].dev->contiguous(keys_c.p, {1, H, T, D}, {max_seq * dim, D, dim, 1}, 0, (size_t)T * dim);
             cache_v[l].dev->contiguous(values_c.p, {1, H, D, T}, {max_seq * dim, D, 1, dim}, 0, (size_t)T * dim);
@@ -297,6 +306,7 @@ struct tlm_model {
             ck(tl_matmul2d_batched_f16(scores.p, values_c.p, s_v.p, S, D, T, H, (size_t)S * T, (size_t)D * T, (size_t)S * D),
                "scores.values");
             s_v.dev->contiguous(o_c.p, {1, S, H, D}, {H * S * D, D, S * D, 1}, 0, sd);
+            }
             matmul2d(o_c.p, w.wo, x_norm.p, S, dim, dim);
             ck(tl_add_rms_norm_f16(x_residual.p, x_norm.p, x.p, x_norm.p, w.ffn_norm, eps, dim, S), "add_rms_norm");
             if (w.w3 == w.w1 + (size_t)hidden * dim && hidden % 8 == 0) {
@@ -382,7 +392,7 @@ int tlm_create(tlm_model** out, int dim, int hidden_dim, int n_layers, int n_hea
         m->scores.alloc(sc); m->scores2.alloc(sc); m->mask.alloc(sc);
         m->xq_c.alloc(sd); m->s_v.alloc(sd); m->o_c.alloc(sd);
         m->keys_c.alloc((size_t)max_seq_len * dim);
-        m->values_c.alloc((size_t)max_seq_len * dim);
+        m->values_c.alloc((size_t)((max_seq_len + 31) / 32 * 32) * dim);   // rows padded for the prefill attention
         m->logits.alloc(S * vocab_size);
         m->rope_table.alloc((size_t)max_seq_len * (dim / n_heads));
         ck(tl_rope_table_f16(m->rope_table.p, max_seq_len, dim / n_heads), "rope_table");
