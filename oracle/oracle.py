@@ -176,6 +176,28 @@ def silu_mul(a: np.ndarray, b: np.ndarray) -> np.ndarray:
     return out
 
 
+def attention_chain(q: np.ndarray, cache_k: np.ndarray, cache_v: np.ndarray, start_pos: int) -> np.ndarray:
+    """Attention::forward after RoPE, composed from the CPU ops one for one
+    (model/llama2_7b/src/Transformer.cpp:61-109): per head matmul2d(q, keys), ScalarDiv by
+    half(sqrt(head_dim)), mask EwiseAdd (only when more than one token, Transformer.cpp:234), softmax(3),
+    matmul2d(scores, values^T).  q: [H, S, D] rotated; caches [>= start_pos + S, H, D].
+    Returns [S, H, D]."""
+    q = _h(q)
+    H, S, D = q.shape
+    T = start_pos + S
+    div = np.float16(np.sqrt(np.float32(D)))
+    mask = np.where(np.arange(T)[None, :] > start_pos + np.arange(S)[:, None], -np.inf, 0.0).astype(np.float16)
+    out = np.empty((S, H, D), np.float16)
+    for h in range(H):
+        k = np.ascontiguousarray(cache_k[:T, h, :])
+        vt = np.ascontiguousarray(cache_v[:T, h, :].T)
+        sc = binary_scalar(matmul2d(np.ascontiguousarray(q[h]), k), div, "div")
+        if S > 1:
+            sc = binary(sc, mask, "add")
+        out[:, h, :] = matmul2d(softmax(sc), vt)
+    return out
+
+
 def _ints(v):
     return (ctypes.c_int * len(v))(*[int(i) for i in v])
 

@@ -45,6 +45,20 @@ def build():
     for op in ("add", "sub", "mul", "div"):
         v["bin_" + op] = o.binary(a, b, op)
     v["div_scalar"] = o.binary_scalar(a, np.float16(11.3125), "div")
+    # attention (after RoPE): prefill of 40 tokens at position 5, and one decode row at position 45
+    H, S, D, start = 2, 40, 64, 5
+    q = synth.normal_f16(12, (H, S, D), 1.0)
+    ck, cv = synth.normal_f16(13, (64, H, D), 1.0), synth.normal_f16(14, (64, H, D), 1.0)
+    v["att_q"], v["att_k"], v["att_v"], v["att_start"] = q, ck, cv, np.array(start)
+    v["att_prefill_y"] = o.attention_chain(q, ck, cv, start)
+    q1 = synth.normal_f16(15, (H, 1, D), 1.0)
+    v["att_q1"], v["att_decode_y"] = q1, o.attention_chain(q1, ck, cv, 45)
+    # residual add -> RMSNorm -> projection (the chain the fused GEMV prologue replaces)
+    hh, dd, gg = synth.normal_f16(16, (1, 512), 1.0), synth.normal_f16(17, (1, 512), 0.7), synth.normal_f16(18, (512,), 1.0)
+    Wn = synth.normal_f16(19, (48, 512), 0.05)
+    sm = o.binary(hh, dd, "add")
+    v["nrm_h"], v["nrm_d"], v["nrm_g"], v["nrm_W"] = hh, dd, gg, Wn
+    v["nrm_sum"], v["nrm_y"] = sm, o.matmul2d(o.rms_norm(sm, gg, 1e-5, "exact"), Wn)
     am = synth.normal_f16(11, (6, 300), 1.0)
     v["argmax_x"], v["argmax_y"] = am, o.argmax(am)
     return v

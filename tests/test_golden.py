@@ -35,6 +35,11 @@ def test_oracle_reproduces_golden_vectors(oracle, gold):
         assert _same(oracle.binary(g["ew_a"], g["ew_b"], op), g["bin_" + op]), op
     assert _same(oracle.binary_scalar(g["ew_a"], np.float16(11.3125), "div"), g["div_scalar"])
     assert np.array_equal(oracle.argmax(g["argmax_x"]), g["argmax_y"])
+    assert _same(oracle.attention_chain(g["att_q"], g["att_k"], g["att_v"], int(g["att_start"])), g["att_prefill_y"])
+    assert _same(oracle.attention_chain(g["att_q1"], g["att_k"], g["att_v"], 45), g["att_decode_y"])
+    sm = oracle.binary(g["nrm_h"], g["nrm_d"], "add")
+    assert _same(sm, g["nrm_sum"])
+    assert _same(oracle.matmul2d(oracle.rms_norm(sm, g["nrm_g"], 1e-5, "exact"), g["nrm_W"]), g["nrm_y"])
 
 
 def test_synthetic_inputs_are_stable(gold):
@@ -62,3 +67,19 @@ def test_gpu_matches_golden_vectors(dev, gold):
         assert _same(dev.binary(up(g["ew_a"]), up(g["ew_b"]), op).cpu().numpy(), g["bin_" + op]), op
     assert _same(dev.div(up(g["ew_a"]), 11.3125).cpu().numpy(), g["div_scalar"])
     assert np.array_equal(dev.argmax(up(g["argmax_x"])).cpu().numpy(), g["argmax_y"])
+
+
+@pytest.mark.gpu
+def test_gpu_fused_kernels_match_golden_chains(dev, gold):
+    """The fused kernels against the frozen outputs of the CPU op chains they replace."""
+    from tests.conftest import assert_close_scaled
+    g = gold
+    up = dev.from_numpy
+    start = int(g["att_start"])
+    got = dev.prefill_attention(up(g["att_q"]), up(g["att_k"]), up(g["att_v"]), start).cpu().numpy()
+    assert_close_f16(got, g["att_prefill_y"], 1e-2, 3e-3, "prefill attention")
+    got = dev.decode_attention(up(np.ascontiguousarray(g["att_q1"][:, 0, :])), up(g["att_k"]), up(g["att_v"]), 46).cpu().numpy()
+    assert_close_f16(got, g["att_decode_y"][0], 1e-2, 2e-3, "decode attention")
+    y, s = dev.gemv_add_rms_norm(up(g["nrm_h"][0]), up(g["nrm_d"][0]), up(g["nrm_g"]), 1e-5, up(g["nrm_W"]))
+    assert _same(s.cpu().numpy(), g["nrm_sum"][0])
+    assert_close_scaled(y.cpu().numpy(), g["nrm_y"][0], 1e-2, 5e-3, "gemv with add + rmsnorm prologue")

@@ -404,22 +404,6 @@ def test_silu_mul_rows(dev, oracle, rows, hidden):
     assert np.array_equal(got.view(np.uint16), two.cpu().numpy().view(np.uint16))
 
 
-def _prefill_attention_oracle(oracle, q, ck, cv, start):
-    """Attention::forward for S new tokens with the CPU ops: per-head matmul2d, ScalarDiv, mask add, softmax, matmul2d."""
-    H, S, D = q.shape
-    T = start + S
-    div = np.float16(np.sqrt(np.float32(D)))
-    mask = np.where(np.arange(T)[None, :] > start + np.arange(S)[:, None], -np.inf, 0.0).astype(np.float16)
-    out = np.empty((S, H, D), np.float16)
-    for h in range(H):
-        k = np.ascontiguousarray(ck[:T, h, :])
-        vt = np.ascontiguousarray(cv[:T, h, :].T)
-        sc = oracle.matmul2d(np.ascontiguousarray(q[h]), k)
-        sc = oracle.binary(oracle.binary_scalar(sc, div, "div"), mask, "add")
-        out[:, h, :] = oracle.matmul2d(oracle.softmax(sc), vt)
-    return out
-
-
 @pytest.mark.parametrize("H,S,D,start", [(4, 128, 128, 0), (2, 70, 128, 9), (3, 33, 64, 100), (2, 1, 128, 40),
                                          (1, 32, 128, 0), (8, 512, 128, 0), (2, 200, 64, 313)])
 def test_prefill_attention(dev, oracle, H, S, D, start):
@@ -428,7 +412,7 @@ def test_prefill_attention(dev, oracle, H, S, D, start):
     q = synth.normal_f16(190, (H, S, D), 1.0)
     ck = synth.normal_f16(191, (T + 3, H, D), 1.0)
     cv = synth.normal_f16(192, (T + 3, H, D), 1.0)
-    want = _prefill_attention_oracle(oracle, q, ck, cv, start)
+    want = oracle.attention_chain(q, ck, cv, start)
     got = dev.prefill_attention(dev.from_numpy(q), dev.from_numpy(ck), dev.from_numpy(cv), start).cpu().numpy()
     # probabilities are rounded to fp16 before (CPU: after) normalisation: a few fp16 ulps on outputs of size ~1
     assert_close_f16(got, want, RTOL, 3e-3, f"prefill attention H={H} S={S} D={D} start={start}")
