@@ -325,3 +325,27 @@ def test_embedding_is_a_row_gather(oracle):
     t = synth.normal_f16(90, (20, 12), 1.0)
     ids = np.array([3, 3, 19, 0], np.int32)
     assert np.array_equal(oracle.embedding(t, ids).view(np.uint16), t[ids].view(np.uint16))
+
+
+# ------------------------------------------------------------------ composed chains ----
+
+def test_attention_chain_against_float64(oracle):
+    """The composed attention chain (per-head matmul2d, ScalarDiv, mask, softmax, matmul2d) against the
+    textbook causal attention in float64: catches a transposed operand, a wrong mask edge or scale."""
+    H, S, D, start = 3, 7, 32, 4
+    T = start + S
+    q = synth.normal_f16(300, (H, S, D), 1.0)
+    ck = synth.normal_f16(301, (T + 2, H, D), 1.0)
+    cv = synth.normal_f16(302, (T + 2, H, D), 1.0)
+    got = oracle.attention_chain(q, ck, cv, start).astype(np.float64)
+    k = ck[:T].astype(np.float64).transpose(1, 0, 2)          # [H, T, D]
+    v = cv[:T].astype(np.float64).transpose(1, 0, 2)
+    sc = np.einsum("hsd,htd->hst", q.astype(np.float64), k) / np.sqrt(D)
+    sc = np.where(np.arange(T)[None, None, :] > start + np.arange(S)[None, :, None], -np.inf, sc)
+    want = np.einsum("hst,htd->shd", scipy_softmax(sc, axis=-1), v)
+    assert np.abs(got - want).max() < 6e-3
+    # a single new token sees every cached position: no mask is applied (Transformer.cpp:234)
+    got1 = oracle.attention_chain(q[:, :1], ck, cv, T - 1).astype(np.float64)
+    sc1 = np.einsum("hsd,htd->hst", q[:, :1].astype(np.float64), k) / np.sqrt(D)
+    want1 = np.einsum("hst,htd->shd", scipy_softmax(sc1, axis=-1), v)
+    assert np.abs(got1 - want1).max() < 6e-3
