@@ -112,6 +112,9 @@ const char* tl_hgemm_variant_name(int variant);
 int tl_measure_mfma_rate_f16(int mode, double* tflops);
 /* Tuning hook: force the number of K splits of the MFMA GEMM (0 = automatic). */
 int tl_set_hgemm_splits(int splits);
+/* Tuning hook: the MFMA GEMM's workgroups start their walk over K at K tile
+ * (tile_column * per_tile + xcd * per_xcd) % tiles and wrap (-1 = automatic, 0 = no rotation). */
+int tl_set_hgemm_k_rotation(int per_tile, int per_xcd);
 /* Tuning hook: cap the GEMV grid at `waves` resident wavefronts per compute unit (0 = default). */
 int tl_set_gemv_grid_waves_per_cu(int waves);
 

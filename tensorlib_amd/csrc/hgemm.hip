@@ -18,6 +18,7 @@
 // in distinct bank groups) and zero-fills the K tail.  gemm_generic_kernel covers everything else.
 #include <cstring>
 #include <mutex>
+#include <numeric>
 #include <type_traits>
 
 #include "tl_internal.h"
@@ -35,6 +36,10 @@ struct HgemmArgs {
     // fp32 partial sums to partial[z][M][N]; a second kernel adds the splits in order.
     int kt_per_split;
     float* partial;
+    // K rotation: a workgroup walks its K tiles starting at (tile_n * rot_tile + xcd * rot_xcd) % KT and wraps.
+    // Workgroups that run at the same time then touch different column offsets of the 8 KB-strided rows, which
+    // spreads their requests over the memory channels (tile-shaped streaming of B from HBM: 4.3 -> 5.9 TB/s).
+    int rot_tile, rot_xcd;
 };
 
 constexpr int kPad = 8;  // halves of padding per LDS row
@@ -259,7 +264,8 @@ __global__ void __launch_bounds__(WM* WN * 64) hgemm_f16_dlds_kernel(HgemmArgs a
     // loop would make the compiler treat lgkmcnt as unordered and turn every wait for LDS data into
     // lgkmcnt(0), which also waits for the fragment reads issued just before it.
     float* const partial = a.partial;
-    asm volatile("" ::"s"(partial), "s"(C), "s"(M), "s"(N), "s"(a.kt_per_split));
+    const unsigned rot_tile = (unsigned)a.rot_tile, rot_xcd = (unsigned)a.rot_xcd;
+    asm volatile("" ::"s"(partial), "s"(C), "s"(M), "s"(N), "s"(a.kt_per_split), "s"(rot_tile), "s"(rot_xcd));
 
     // ---- loader: wavefront-load j of this wavefront covers tile rows (j*NW + wave)*RPW .. +RPW ----
     const int ld_row_in_group = lane / CPR;
@@ -270,11 +276,13 @@ __global__ void __launch_bounds__(WM* WN * 64) hgemm_f16_dlds_kernel(HgemmArgs a
     const int kt_begin = (int)blockIdx.z * a.kt_per_split;
     const int KT = (KT_all - kt_begin) < a.kt_per_split ? (KT_all - kt_begin) : a.kt_per_split;
     // tile `b` of the launch: sets m0, n0 and the per-lane source pointers (at this split's first K tile)
+    int rot = 0;  // first K tile of this workgroup's walk (relative to its split)
     auto setup_tile = [&](int b) {
         int tile_m, tile_n;
         tile_of_block(b, total_tiles, a.tiles_m, tile_m, tile_n);
         m0 = tile_m * BM;
         n0 = tile_n * BN;
+        rot = KT > 0 ? (int)(((unsigned)tile_n * rot_tile + (blockIdx.x & 7u) * rot_xcd) % (unsigned)KT) : 0;
 #pragma unroll
         for (int j = 0; j < A_LOADS; ++j) {
             const int r = (j * NW + wave) * RPW + ld_row_in_group;  // tile row
@@ -296,23 +304,29 @@ __global__ void __launch_bounds__(WM* WN * 64) hgemm_f16_dlds_kernel(HgemmArgs a
     setup_tile(vb);
     auto a_off = [&](int kt) { return (kt % STAGES) * STAGE_BYTES; };
     auto b_off = [&](int kt) { return (kt % STAGES) * STAGE_BYTES + A_BYTES; };
+    // element offset of the kt-th K tile of the walk
+    auto k_of = [&](int kt) {
+        int k = kt + rot;
+        k = k >= KT ? k - KT : k;
+        return (size_t)k * BK;
+    };
     auto issue_a = [&](int kt) {
         lds_byte_t* sa = lds + a_off(kt);
-        const size_t koff = (size_t)kt * BK;
+        const size_t koff = k_of(kt);
 #pragma unroll
         for (int j = 0; j < A_LOADS; ++j)
             load_16B_per_lane_to_lds(a_src[j] + koff, sa + (j * NW + wave) * 1024);
     };
     auto issue_b = [&](int kt) {
         lds_byte_t* sb = lds + b_off(kt);
-        const size_t koff = (size_t)kt * BK;
+        const size_t koff = k_of(kt);
 #pragma unroll
         for (int j = 0; j < B_LOADS; ++j)
             load_16B_per_lane_to_lds(b_src[j] + koff, sb + (j * NW + wave) * 1024);
     };
     // wavefront-load l of tile kt: l < A_LOADS from A, the rest from B
     auto issue_one = [&](int kt, int l) {
-        const size_t koff = (size_t)kt * BK;
+        const size_t koff = k_of(kt);
         if (l < A_LOADS)
             load_16B_per_lane_to_lds(a_src[l] + koff, lds + a_off(kt) + (l * NW + wave) * 1024);
         else
@@ -635,6 +649,7 @@ static int g_forced_variant = 0;
 static bool g_attr_set[kNumVariants] = {false};
 
 static int g_forced_splits = 0;  // 0 = automatic
+static int g_forced_rot_tile = -1, g_forced_rot_xcd = -1;  // -1 = automatic
 
 // Library-owned fp32 workspace for split-K partial sums, grown on demand (stream-ordered reuse).
 static std::mutex g_ws_mu;
@@ -763,6 +778,8 @@ int launch_hgemm(const void* A, const void* B, void* C, size_t M, size_t N, size
     TL_REQUIRE(nblocks <= 0x7fffffffu, "hgemm: too many tiles");
     a.kt_per_split = 0x7fffffff;
     a.partial = nullptr;
+    a.rot_tile = 0;
+    a.rot_xcd = 0;
     int splits = 1;
     if (v.stages > 0) {
         // Split K when the tile grid alone cannot occupy the chip (prefill with few tokens: the
@@ -794,6 +811,19 @@ int launch_hgemm(const void* A, const void* B, void* C, size_t M, size_t N, size
     if (v.stages <= 3 && v.name[0] == 'p') {
         const size_t resident = (size_t)device_info().cu_count * ((160 * 1024) / lds > 0 ? (160 * 1024) / lds : 1);
         if (grid_x > resident) grid_x = resident;
+    }
+    if (v.stages > 0) {
+        const int KT = (int)(K / v.bk);
+        const int kt_walk = a.kt_per_split < KT ? a.kt_per_split : KT;
+        if (M <= 512) {
+            // rows of B are private to a column of tiles: spread the tiles over the K offsets
+            for (int c : {5, 7, 11, 13, 3, 1})
+                if (std::gcd(c, kt_walk) == 1) { a.rot_tile = c; break; }
+        } else {
+            a.rot_xcd = kt_walk / 8;  // tiles of one XCD keep walking K together (they share panels through its L2)
+        }
+        if (g_forced_rot_tile >= 0) a.rot_tile = g_forced_rot_tile;
+        if (g_forced_rot_xcd >= 0) a.rot_xcd = g_forced_rot_xcd;
     }
     hipLaunchKernelGGL(v.kernel, dim3((unsigned)grid_x, (unsigned)batch, (unsigned)splits), dim3(v.threads), lds, st, a);
     TL_CHECK_LAUNCH(v.name);
@@ -858,6 +888,13 @@ int tl_set_hgemm_variant(int variant) {
 int tl_set_hgemm_splits(int splits) {
     TL_REQUIRE(splits >= 0 && splits <= 64, "tl_set_hgemm_splits: %d out of range [0,64]", splits);
     tl::g_forced_splits = splits;
+    return TL_OK;
+}
+
+int tl_set_hgemm_k_rotation(int per_tile, int per_xcd) {
+    TL_REQUIRE(per_tile >= -1 && per_xcd >= -1, "tl_set_hgemm_k_rotation: negative step");
+    tl::g_forced_rot_tile = per_tile;
+    tl::g_forced_rot_xcd = per_xcd;
     return TL_OK;
 }
 

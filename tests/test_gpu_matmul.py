@@ -159,6 +159,30 @@ def test_hgemm_integer_inputs_bit_exact(dev, oracle):
     assert np.array_equal(C.astype(np.float64), ref)
 
 
+def test_hgemm_k_rotation_and_splits_visit_every_k_tile_once(dev, oracle):
+    """Workgroups start their walk over K at a rotated tile and wrap, per split: with small-integer data the
+    result is exact whatever the order, so a skipped or repeated K tile shows as a wrong bit."""
+    names = dev.hgemm_variants()
+    try:
+        for (M, N, K) in [(128, 640, 448), (300, 1100, 704), (512, 2112, 1024)]:
+            A = synth.small_ints_f16(1250 + K, (M, K), -2, 2)
+            B = synth.small_ints_f16(1251 + K, (N, K), -2, 2)
+            want = oracle.matmul2d(A, B).view(np.uint16)
+            Ad, Bd = dev.from_numpy(A), dev.from_numpy(B)
+            for name in ("auto", "p256x256x64w2x4s2", "p128x128x64w2x4s4", "p128x64x64w4x1s4"):
+                dev.set_hgemm_variant(names.index(name))
+                for splits in (0, 1, 3):
+                    dev.lib.tl_set_hgemm_splits(splits)
+                    for rot in ((-1, -1), (0, 0), (1, 0), (5, 3), (0, 2), (1000003, 17)):
+                        dev.lib.tl_set_hgemm_k_rotation(*rot)
+                        C = dev.hgemm(Ad, Bd).cpu().numpy()
+                        assert np.array_equal(C.view(np.uint16), want), (M, N, K, name, splits, rot)
+    finally:
+        dev.set_hgemm_variant(0)
+        dev.lib.tl_set_hgemm_splits(0)
+        dev.lib.tl_set_hgemm_k_rotation(-1, -1)
+
+
 def test_hgemm_identity(dev):
     """B = I returns A; A = I returns B^T (catches a transposed operand or tile mapping)."""
     n = 320
