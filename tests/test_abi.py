@@ -39,6 +39,17 @@ def test_llama2_driver_exports_its_header():
     assert not [s for s in declared if not hasattr(handle, s)]
 
 
+def test_tokenizer_exports_its_header():
+    from tensorlib_amd import llama2, tokenizer
+    text = open(os.path.join(ROOT, "include", "tensorlib_tokenizer.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    declared = sorted(set(re.findall(r"\b(tlt_[a-z0-9_]+)\s*\(", text)))
+    assert sorted(tokenizer._PROTOS) == declared
+    ctypes.CDLL(_lib.LIB_PATH, mode=ctypes.RTLD_GLOBAL)
+    handle = ctypes.CDLL(llama2.LLAMA2_LIB_PATH)
+    assert not [s for s in declared if not hasattr(handle, s)]
+
+
 def test_header_cites_the_reference_for_each_hot_path_entry():
     text = open(_lib.HEADER).read()
     for sym in ["tl_matmul2d_f16", "tl_gemv_f16", "tl_hgemm_f16", "tl_rms_norm_f16", "tl_apply_rotary_emb_f16",
