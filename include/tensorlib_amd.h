@@ -115,6 +115,9 @@ int tl_set_hgemm_splits(int splits);
 /* Tuning hook: the MFMA GEMM's workgroups start their walk over K at K tile
  * (tile_column * per_tile + xcd * per_xcd) % tiles and wrap (-1 = automatic, 0 = no rotation). */
 int tl_set_hgemm_k_rotation(int per_tile, int per_xcd);
+/* Tuning hook: prefill attention kernel, 0 = automatic, 1 = one wavefront per 32 query rows,
+ * 2 = LDS-tiled workgroups of 128 query rows (head_dim 128, ldv covering the context rounded up to 64). */
+int tl_set_prefill_attention_variant(int variant);
 /* Tuning hook: cap the GEMV grid at `waves` resident wavefronts per compute unit (0 = default). */
 int tl_set_gemv_grid_waves_per_cu(int waves);
 
@@ -242,7 +245,8 @@ int tl_gather_vt_f16(void* vT, const void* cache_v, int T, int ldv, int n_heads,
  * (Attention::forward, model/llama2_7b/src/Transformer.cpp:92-109) without a score matrix in memory.
  * q: [n_heads, n_tokens, head_dim] (rotated, as tl_prefill_rope_qkv_f16 writes it); cache_k: [.., n_heads,
  * head_dim]; vT from tl_gather_vt_f16 with ldv >= the context rounded up to 32; out: [n_tokens, n_heads,
- * head_dim].  head_dim 64 or 128. */
+ * head_dim].  head_dim 64 or 128.  With head_dim 128, at least 128 new tokens and ldv >= the context rounded up
+ * to 64, workgroups of 128 query rows share key tiles through LDS (same results bit for bit). */
 int tl_prefill_attention_f16(void* out, const void* q, const void* cache_k, const void* vT, int ldv, int start_pos,
                              int n_tokens, int n_heads, int head_dim);
 

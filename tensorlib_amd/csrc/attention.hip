@@ -17,6 +17,9 @@
 
 namespace tl {
 
+// 0: automatic, 1: one wavefront per 32 query rows, 2: LDS-tiled workgroups of 128 query rows (tuning hook)
+static int g_prefill_attention_variant = 0;
+
 template <int CTRL>
 __device__ __forceinline__ float dppf(float v) {
     return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, true));
@@ -297,12 +300,68 @@ gather_vt_kernel(half_t* vT, const half_t* cache_v, int T, int ldv, int n_heads,
     }
 }
 
+// Scores of one block of 32 keys x 32 query rows -> probabilities, online-softmax state update.
+// sacc[4g + r] of lane (lr, lh) is the fp32 score of key t0 + 8g + 4*lh + r against the lane's query row.
+// Rounding follows the reference chain: score to fp16, fp16 quotient by half(sqrt(head_dim)) (the quotient
+// is formed as x*r corrected by one fused Newton step, which rounds to the same fp16 value as the fp32
+// division for every fp16 x and both supported divisors; exhaustively checked on the host), -inf above the
+// diagonal (MASK: only blocks that reach the diagonal pay for it), exp in fp32, probability to fp16 (summed by attn_add_row_sums).
+// The softmax is bound by vector-ALU instructions (1024 scores per 16 MFMAs), so the work per score is kept
+// to conversions the hardware fuses into fma_mix, a packed-fp16 maximum, one fma + exp2 and the fp32 sum.
+// The row maximum is finite from the first block on (key 0 is visible to every query), so exp2(-inf) = 0
+// covers the first block without a guard.  Returns the factor by which the running output is to be rescaled
+// (1 when the maximum did not move).
+template <bool MASK>
+__device__ __forceinline__ float attn_block_softmax(const float16_t& sacc, int t0, int lh, int limit, float dv,
+                                                    float rdv, float& m, half8_t (&pf)[2]) {
+    constexpr float kLog2e = 1.4426950408889634f;
+    half_t sh[16];
+#pragma unroll
+    for (int e = 0; e < 16; ++e) {
+        const half_t xh = (half_t)sacc[e];
+        const float qv = (float)xh * rdv;
+        sh[e] = (half_t)__builtin_fmaf(__builtin_fmaf(-qv, dv, (float)xh), rdv, qv);
+        if constexpr (MASK) {
+            const int kk = t0 + 8 * (e / 4) + 4 * lh + (e % 4);
+            sh[e] = kk <= limit ? sh[e] : (half_t)-INFINITY;
+        }
+    }
+    half2_t mx = {sh[0], sh[1]};
+#pragma unroll
+    for (int e = 2; e < 16; e += 2) {
+        const half2_t t = {sh[e], sh[e + 1]};
+        mx = __builtin_elementwise_max(mx, t);
+    }
+    float bm = (float)(mx[0] > mx[1] ? mx[0] : mx[1]);
+    bm = fmaxf(bm, __shfl_xor(bm, 32, 64));
+    const float m_new = fmaxf(m, bm);
+    const float corr = __builtin_amdgcn_exp2f((m - m_new) * kLog2e);
+    const float nm = -m_new * kLog2e;
+#pragma unroll
+    for (int e = 0; e < 16; ++e)      // MFMA step s = e / 8 holds g = 2s (slots 0..3) and g = 2s + 1 (slots 4..7)
+        pf[e / 8][e % 8] = (half_t)__builtin_amdgcn_exp2f(__builtin_fmaf((float)sh[e], kLog2e, nm));
+    m = m_new;
+    return corr;
+}
+
+// Row sums of the fp16 probabilities of a block, added to the running sums: an MFMA whose A operand is all
+// ones leaves sum_key P^T[key][q] in every row of column q, i.e. in element 0 of both lanes that own query
+// row q (the matrix core is idle while the softmax runs; a vector-ALU sum costs 32 instructions and a lane
+// exchange).  Only element 0 is kept meaningful: it alone is rescaled.
+__device__ __forceinline__ void attn_add_row_sums(float16_t& lacc, const half8_t (&pf)[2], float corr, bool rescale) {
+    const half8_t ones = {(half_t)1.f, (half_t)1.f, (half_t)1.f, (half_t)1.f, (half_t)1.f, (half_t)1.f, (half_t)1.f, (half_t)1.f};
+    if (rescale) lacc[0] *= corr;
+    lacc = __builtin_amdgcn_mfma_f32_32x32x16_f16(ones, pf[0], lacc, 0, 0, 0);
+    lacc = __builtin_amdgcn_mfma_f32_32x32x16_f16(ones, pf[1], lacc, 0, 0, 0);
+}
+
 // Causal attention of n_tokens new tokens against cache positions [0, start_pos + n_tokens): one wavefront per
 // (head, 32 query rows), no LDS, no score matrix in memory.  Per block of 32 keys:
 //   S^T[key][q] = sum_d K[key][d] Q[q][d]        8 MFMAs, A = K rows straight from the cache, B = Q (registers)
-//   lane l then holds 16 keys of ONE query row (l % 32): the online-softmax row reductions are in-lane plus
-//   one exchange with lane l ^ 32; scores are rounded like the reference chain (fp16 score, fp16 quotient by
-//   half(sqrt(head_dim)), -inf above the diagonal);
+//   lane l then holds 16 keys of ONE query row (l % 32): the row maximum is in-lane plus one exchange with
+//   lane l ^ 32; scores are rounded like the reference chain (fp16 score, fp16 quotient by
+//   half(sqrt(head_dim)), -inf above the diagonal); the row sums of the fp16 probabilities come from an MFMA
+//   with an all-ones operand;
 //   O^T[d][q] += sum_key vT[d][key] P^T[key][q]   A = vT with the key order the accumulator layout dictates
 //   (lane half h of MFMA step s owns keys 16s+4h+{0..3} and 16s+8+4h+{0..3}: two 8-byte loads), B = P^T taken
 //   from the score accumulators of the same lane without any shuffle.
@@ -326,7 +385,7 @@ prefill_attention_kernel(half_t* out, const half_t* q, const half_t* cache_k, co
     const int my_q = q0 + lr;                       // the query row this lane owns in S^T / O^T
     const int my_q_c = my_q < n_tokens ? my_q : n_tokens - 1;
     const int limit = start_pos + my_q;             // last visible key
-    const float dv = (float)divisor;
+    const float dv = (float)divisor, rdv = 1.0f / dv;
 
     half8_t qf[KS];
     const half_t* qrow = q + ((size_t)h * n_tokens + my_q_c) * D + lh * 8;
@@ -338,7 +397,10 @@ prefill_attention_kernel(half_t* out, const half_t* q, const half_t* cache_k, co
     for (int b = 0; b < DB; ++b)
 #pragma unroll
         for (int e = 0; e < 16; ++e) o[b][e] = 0.f;
-    float m = -INFINITY, l = 0.f;
+    float m = -INFINITY;
+    float16_t lacc;
+#pragma unroll
+    for (int e = 0; e < 16; ++e) lacc[e] = 0.f;
 
     const int last_key = start_pos + (q0 + 31 < n_tokens ? q0 + 31 : n_tokens - 1);  // of the whole wavefront
     const size_t krow_stride = (size_t)n_heads * D;
@@ -370,37 +432,18 @@ prefill_attention_kernel(half_t* out, const half_t* q, const half_t* cache_k, co
         for (int e = 0; e < 16; ++e) sacc[e] = 0.f;
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) sacc = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf[ks], qf[ks], sacc, 0, 0, 0);
-        // sacc[4g + r] = score of key t0 + 8g + 4*lh + r against query my_q
-        float sv[16];
-        float bm = -INFINITY;
-#pragma unroll
-        for (int e = 0; e < 16; ++e) {
-            const int kk = t0 + 8 * (e / 4) + 4 * lh + (e % 4);
-            const half_t s16 = (half_t)sacc[e];
-            const float t = (float)(half_t)((float)s16 / dv);
-            sv[e] = kk <= limit ? t : -INFINITY;
-            bm = fmaxf(bm, sv[e]);
-        }
-        bm = fmaxf(bm, __shfl_xor(bm, 32, 64));
-        const float m_new = fmaxf(m, bm);
-        const float corr = (m == -INFINITY) ? 0.f : expf(m - m_new);
-        float bs = 0.f;
         half8_t pf[2];
-#pragma unroll
-        for (int e = 0; e < 16; ++e) {
-            const float pv = (m_new == -INFINITY) ? 0.f : expf(sv[e] - m_new);
-            const half_t p16 = (half_t)pv;
-            bs += (float)p16;
-            pf[e / 8][e % 8] = p16;       // step s = e / 8 holds g = 2s (slots 0..3) and g = 2s + 1 (slots 4..7)
-        }
-        bs += __shfl_xor(bs, 32, 64);
-        l = l * corr + bs;
-        m = m_new;
+        const float corr = t0 + 31 > start_pos + q0 ? attn_block_softmax<true>(sacc, t0, lh, limit, dv, rdv, m, pf)
+                                                    : attn_block_softmax<false>(sacc, t0, lh, limit, dv, rdv, m, pf);
+        const bool rescale = __builtin_amdgcn_ballot_w64(corr != 1.0f) != 0;
+        attn_add_row_sums(lacc, pf, corr, rescale);
         // ---- O^T += vT . P^T ----
 #pragma unroll
         for (int b = 0; b < DB; ++b) {
+            if (rescale) {
 #pragma unroll
-            for (int e = 0; e < 16; ++e) o[b][e] *= corr;
+                for (int e = 0; e < 16; ++e) o[b][e] *= corr;
+            }
 #pragma unroll
             for (int st = 0; st < 2; ++st) {
                 const half4_t v0 = vraw[b][st][0], v1 = vraw[b][st][1];
@@ -412,7 +455,7 @@ prefill_attention_kernel(half_t* out, const half_t* q, const half_t* cache_k, co
         for (int ks = 0; ks < KS; ++ks) kf[ks] = kn[ks];
     }
     if (my_q >= n_tokens) return;
-    const float inv = 1.0f / l;
+    const float inv = 1.0f / lacc[0];
     half_t* orow = out + ((size_t)my_q * n_heads + h) * D;
 #pragma unroll
     for (int b = 0; b < DB; ++b)
@@ -422,6 +465,176 @@ prefill_attention_kernel(half_t* out, const half_t* q, const half_t* cache_k, co
                          (half_t)(o[b][4 * g + 3] * inv)};
             *reinterpret_cast<half4_t*>(orow + b * 32 + 8 * g + 4 * lh) = r;
         }
+}
+
+// The same attention for long prompts: a workgroup of four wavefronts owns 128 query rows of one head and
+// walks the keys in tiles of 64, K rows and vT rows of a tile staged once in LDS (direct global->LDS loads, two
+// stages) and read from there by all four wavefronts.  Per wavefront and block of 32 keys the arithmetic and
+// its order are exactly those of prefill_attention_kernel (results are bit-identical); what changes is the
+// traffic: that kernel re-reads a head's K and V for every 32 query rows (1.1 GB per layer at 2048 tokens),
+// this one for every 128.  LDS layout, 16-byte chunks swizzled so that the 16 rows one ds_read phase touches
+// fall into different banks: K tile [64 keys][256 B], chunk c of row r at slot c ^ (r % 16); vT tile
+// [128 d][128 B], chunk c of row r at slot c ^ ((r / 2) % 8).  Needs vT rows that cover the context rounded up
+// to 64.
+// Registers are capped for two workgroups per CU (each hides the other's barriers and softmax); the cap also gave
+// the faster code when only one is resident.
+template <int D, bool PAIRED>
+__global__ void __launch_bounds__(256, 2)
+prefill_attention_tiled_kernel(half_t* out, const half_t* q, const half_t* cache_k, const half_t* vT, int ldv,
+                               int start_pos, int n_tokens, int n_heads, half_t divisor) {
+    static_assert(D == 128, "tile layout is written for head_dim 128");
+    constexpr int KS = D / 16, DB = D / 32, TK = 64, NWQ = 4;
+    constexpr int K_BYTES = TK * D * 2, V_BYTES = D * TK * 2, STAGE_BYTES = K_BYTES + V_BYTES;
+    constexpr int K_LOADS = K_BYTES / 1024 / NWQ, V_LOADS = V_BYTES / 1024 / NWQ;   // wavefront-loads per wavefront
+    extern __shared__ __attribute__((aligned(1024))) unsigned char smem_raw[];
+    typedef __attribute__((address_space(3))) unsigned char lds_byte_t;
+    lds_byte_t* lds = (lds_byte_t*)smem_raw;
+
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int h = blockIdx.y;
+    const int T = start_pos + n_tokens;
+    const int lr = lane & 31, lh = lane >> 5;
+    const float dv = (float)divisor, rdv = 1.0f / dv;
+
+    // loader: K wavefront-load u covers tile rows 4u..4u+3, vT wavefront-load u covers d rows 8u..8u+7
+    const size_t krow_stride = (size_t)n_heads * D;
+    int k_row[K_LOADS], k_chunk[K_LOADS];
+    const half_t* v_src[V_LOADS];
+#pragma unroll
+    for (int j = 0; j < K_LOADS; ++j) {
+        const int u = j * NWQ + wave;
+        k_row[j] = 4 * u + lane / 16;
+        k_chunk[j] = (lane % 16) ^ (k_row[j] % 16);
+    }
+#pragma unroll
+    for (int j = 0; j < V_LOADS; ++j) {
+        const int u = j * NWQ + wave;
+        const int r = 8 * u + lane / 8;
+        const int c = (lane % 8) ^ ((r / 2) % 8);
+        v_src[j] = vT + ((size_t)h * D + r) * ldv + c * 8;
+    }
+    auto issue = [&](int tile, int stage) {
+        const int t0 = tile * TK;
+        lds_byte_t* base = lds + stage * STAGE_BYTES;
+#pragma unroll
+        for (int j = 0; j < K_LOADS; ++j) {
+            int key = t0 + k_row[j];
+            key = key < T ? key : T - 1;
+            load_16B_per_lane_to_lds(cache_k + (size_t)key * krow_stride + (size_t)h * D + k_chunk[j] * 8,
+                                     base + (j * NWQ + wave) * 1024);
+        }
+#pragma unroll
+        for (int j = 0; j < V_LOADS; ++j)
+            load_16B_per_lane_to_lds(v_src[j] + t0, base + K_BYTES + (j * NWQ + wave) * 1024);
+    };
+
+    // Query groups are issued longest first.  With more groups than the chip holds at once (PAIRED) a workgroup
+    // takes two of them, the longest with the shortest, so that every workgroup walks the same number of key
+    // tiles and the kernel does not end on a few long walks.
+    const int n_groups = (n_tokens + 32 * NWQ - 1) / (32 * NWQ);
+    for (int job = 0; job < 2; ++job) {
+        const int group = job == 0 ? n_groups - 1 - (int)blockIdx.x : (int)blockIdx.x;
+        if (job == 1) {
+            if (!PAIRED || group >= n_groups - 1 - (int)blockIdx.x) break;   // odd count: the middle group has no partner
+            asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");   // the stages are free again
+        }
+        const int qg0 = group * (32 * NWQ);                                    // first query row of the group
+        const int q0 = qg0 + 32 * wave;                                       // of this wavefront
+        const int wg_last_key = start_pos + (qg0 + 32 * NWQ - 1 < n_tokens ? qg0 + 32 * NWQ - 1 : n_tokens - 1);
+        const int ntiles = wg_last_key / TK + 1;
+        const bool active = q0 < n_tokens;
+        const int my_q = q0 + lr;
+        const int my_q_c = my_q < n_tokens ? my_q : n_tokens - 1;
+        const int limit = start_pos + my_q;
+        const int last_key = start_pos + (q0 + 31 < n_tokens ? q0 + 31 : n_tokens - 1);
+
+        half8_t qf[KS];
+        const half_t* qrow = q + ((size_t)h * n_tokens + my_q_c) * D + lh * 8;
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) qf[ks] = *reinterpret_cast<const half8_t*>(qrow + ks * 16);
+
+        float16_t o[DB];
+#pragma unroll
+        for (int b = 0; b < DB; ++b)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) o[b][e] = 0.f;
+        float m = -INFINITY;
+        float16_t lacc;
+#pragma unroll
+        for (int e = 0; e < 16; ++e) lacc[e] = 0.f;
+
+        issue(0, 0);
+        if (ntiles > 1) issue(1, 1);
+        for (int i = 0; i < ntiles; ++i) {
+            if (i + 1 < ntiles) wait_vmcnt_and_barrier<K_LOADS + V_LOADS>();
+            else wait_vmcnt_and_barrier<0>();
+            const unsigned char* kt = smem_raw + (i & 1) * STAGE_BYTES;
+            const unsigned char* vt = kt + K_BYTES;
+            if (active && i * TK <= last_key) {
+                // scores of a block: one MFMA per 16 values of head_dim, K fragments read from the swizzled tile
+                auto score_step = [&](float16_t& sacc, int kb, int ks) {
+                    const int kr = 32 * kb + lr;
+                    const half8_t kf = *reinterpret_cast<const half8_t*>(kt + kr * (D * 2) + (((2 * ks + lh) ^ (kr % 16)) * 16));
+                    sacc = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf, qf[ks], sacc, 0, 0, 0);
+                };
+                auto finish_block = [&](const float16_t& sacc, int kb) {
+                    const int t0 = i * TK + 32 * kb;
+                    half8_t pf[2];
+                    const float corr = t0 + 31 > start_pos + q0 ? attn_block_softmax<true>(sacc, t0, lh, limit, dv, rdv, m, pf)
+                                                                : attn_block_softmax<false>(sacc, t0, lh, limit, dv, rdv, m, pf);
+                    const bool rescale = __builtin_amdgcn_ballot_w64(corr != 1.0f) != 0;
+                    attn_add_row_sums(lacc, pf, corr, rescale);
+                    // ---- O^T += vT . P^T ----
+#pragma unroll
+                    for (int b = 0; b < DB; ++b) {
+                        if (rescale) {
+#pragma unroll
+                            for (int e = 0; e < 16; ++e) o[b][e] *= corr;
+                        }
+                        const int vr = 32 * b + lr;
+                        const unsigned char* vrow = vt + vr * (TK * 2) + 8 * lh;
+                        const int sw = (vr / 2) % 8;
+#pragma unroll
+                        for (int st = 0; st < 2; ++st) {
+                            const int c0 = 4 * kb + 2 * st;
+                            const half4_t v0 = *reinterpret_cast<const half4_t*>(vrow + ((c0 ^ sw) * 16));
+                            const half4_t v1 = *reinterpret_cast<const half4_t*>(vrow + (((c0 + 1) ^ sw) * 16));
+                            const half8_t vf = {v0[0], v0[1], v0[2], v0[3], v1[0], v1[1], v1[2], v1[3]};
+                            o[b] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf, pf[st], o[b], 0, 0, 0);
+                        }
+                    }
+                };
+#pragma unroll
+                for (int kb = 0; kb < TK / 32; ++kb) {
+                    if (i * TK + 32 * kb > last_key) break;
+                    float16_t sacc;
+#pragma unroll
+                    for (int e = 0; e < 16; ++e) sacc[e] = 0.f;
+#pragma unroll
+                    for (int ks = 0; ks < KS; ++ks) score_step(sacc, kb, ks);
+                    finish_block(sacc, kb);
+                }
+            }
+            if (i + 2 < ntiles) {
+                // everyone is done reading this stage before the tile after next lands in it
+                asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+                issue(i + 2, i & 1);
+            }
+        }
+        if (active && my_q < n_tokens) {
+            const float inv = 1.0f / lacc[0];
+            half_t* orow = out + ((size_t)my_q * n_heads + h) * D;
+#pragma unroll
+            for (int b = 0; b < DB; ++b)
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    half4_t r = {(half_t)(o[b][4 * g] * inv), (half_t)(o[b][4 * g + 1] * inv), (half_t)(o[b][4 * g + 2] * inv),
+                                 (half_t)(o[b][4 * g + 3] * inv)};
+                    *reinterpret_cast<half4_t*>(orow + b * 32 + 8 * g + 4 * lh) = r;
+                }
+        }
+    }
 }
 
 // Decode-step glue after the fused q|k|v GEMV: rotate q in place, rotate k and write it to
@@ -683,6 +896,29 @@ int tl_prefill_attention_f16(void* out, const void* q, const void* cache_k, cons
                "tl_prefill_attention_f16: operands must be 16-byte aligned");
     const float sq = sqrtf((float)head_dim);
     const tl::half_t divisor = (tl::half_t)sq;  // the reference divides by half(sqrt(head_dim)) (Transformer.cpp:94)
+    const int variant = tl::g_prefill_attention_variant;
+    const bool tiled_ok = head_dim == 128 && ldv >= ((start_pos + n_tokens + 63) / 64) * 64;
+    if (variant == 2) TL_REQUIRE(tiled_ok, "tl_prefill_attention_f16: the tiled kernel needs head_dim 128 and ldv covering the context rounded up to 64");
+    if (tiled_ok && (variant == 2 || (variant == 0 && n_tokens >= 128))) {
+        static bool attr_set = false;
+        constexpr int lds_bytes = 2 * (64 * 128 * 2 + 128 * 64 * 2);
+        if (!attr_set) {
+            TL_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(tl::prefill_attention_tiled_kernel<128, false>),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes));
+            TL_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(tl::prefill_attention_tiled_kernel<128, true>),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes));
+            attr_set = true;
+        }
+        const unsigned groups = (unsigned)((n_tokens + 127) / 128);
+        // two workgroups fit a CU; beyond that a workgroup takes a long and a short group of 128 query rows
+        const bool paired = (size_t)groups * (size_t)n_heads >= 2 * (size_t)tl::device_info().cu_count;
+        dim3 tgrid(paired ? (groups + 1) / 2 : groups, (unsigned)n_heads);
+        auto kernel = paired ? tl::prefill_attention_tiled_kernel<128, true> : tl::prefill_attention_tiled_kernel<128, false>;
+        hipLaunchKernelGGL(kernel, tgrid, dim3(256), lds_bytes, tl::stream(), (tl::half_t*)out, (const tl::half_t*)q,
+                           (const tl::half_t*)cache_k, (const tl::half_t*)vT, ldv, start_pos, n_tokens, n_heads, divisor);
+        TL_CHECK_LAUNCH("prefill_attention_tiled_kernel");
+        return TL_OK;
+    }
     dim3 grid((unsigned)((n_tokens + 31) / 32), (unsigned)n_heads);
     if (head_dim == 64)
         hipLaunchKernelGGL(tl::prefill_attention_kernel<64>, grid, dim3(64), 0, tl::stream(), (tl::half_t*)out,
@@ -693,6 +929,12 @@ int tl_prefill_attention_f16(void* out, const void* q, const void* cache_k, cons
                            (const tl::half_t*)q, (const tl::half_t*)cache_k, (const tl::half_t*)vT, ldv, start_pos, n_tokens,
                            n_heads, divisor);
     TL_CHECK_LAUNCH("prefill_attention_kernel");
+    return TL_OK;
+}
+
+int tl_set_prefill_attention_variant(int variant) {
+    TL_REQUIRE(variant >= 0 && variant <= 2, "tl_set_prefill_attention_variant: %d out of range [0,2]", variant);
+    tl::g_prefill_attention_variant = variant;
     return TL_OK;
 }
 

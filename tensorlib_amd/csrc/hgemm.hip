@@ -198,25 +198,6 @@ __global__ void __launch_bounds__(WM* WN * 64) hgemm_f16_mfma_kernel(HgemmArgs a
 // rows fill one 256-byte LDS line and CPR is the number of chunks per row.  The 16 rows a
 // ds_read_b128 group touches then land in 16 different 16-byte bank groups.
 // Requirements: K % BK == 0 (no zero fill is possible on this path), K % 8 == 0, aligned operands.
-// One global_load_lds_dwordx4: lane l's 16 bytes at `src` go to LDS bytes [dst + 16*l, +16).
-// Written as inline assembly on purpose: the compiler models this instruction as a flat access that may
-// touch LDS, and while one is outstanding (always, in a ring whose vmcnt waits it cannot see) it turns
-// every wait for ds_read data into lgkmcnt(0), including reads issued an instant earlier.  Hidden from
-// it, the ds_reads are the only lgkmcnt traffic and get exact in-order counts.
-__device__ __forceinline__ void load_16B_per_lane_to_lds(const half_t* src,
-                                                         __attribute__((address_space(3))) unsigned char* dst) {
-    const unsigned lds_addr = (unsigned)(unsigned long)dst;
-    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(src), "s"(lds_addr) : "memory");
-}
-
-template <int N_>
-__device__ __forceinline__ void wait_vmcnt_and_barrier() {
-    // waits until at most N_ of this wavefront's global->LDS loads are outstanding and all of its
-    // LDS reads have returned, then joins the workgroup barrier; the "memory" clobber keeps LDS
-    // accesses on their side of it
-    asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(N_) : "memory");
-}
-
 // MODE 0: every wavefront reads the fragments of a K step, then issues its MFMAs.
 // MODE 1: fragments double buffered in registers across K steps.
 template <int BM, int BN, int BK, int WM, int WN, int STAGES, int MODE>

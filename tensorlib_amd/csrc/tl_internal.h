@@ -56,6 +56,27 @@ int launch_hgemm(const void* A, const void* B, void* C, size_t M, size_t N, size
 
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
+#if defined(__HIPCC__)
+// One global_load_lds_dwordx4: lane l's 16 bytes at `src` go to LDS bytes [dst + 16*l, +16).
+// Written as inline assembly on purpose: the compiler models this instruction as a flat access that may
+// touch LDS, and while one is outstanding (always, in a ring whose vmcnt waits it cannot see) it turns
+// every wait for ds_read data into lgkmcnt(0), including reads issued an instant earlier.  Hidden from
+// it, the ds_reads are the only lgkmcnt traffic and get exact in-order counts.
+__device__ __forceinline__ void load_16B_per_lane_to_lds(const half_t* src,
+                                                         __attribute__((address_space(3))) unsigned char* dst) {
+    const unsigned lds_addr = (unsigned)(unsigned long)dst;
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(src), "s"(lds_addr) : "memory");
+}
+
+template <int N_>
+__device__ __forceinline__ void wait_vmcnt_and_barrier() {
+    // waits until at most N_ of this wavefront's global->LDS loads are outstanding and all of its
+    // LDS reads have returned, then joins the workgroup barrier; the "memory" clobber keeps LDS
+    // accesses on their side of it
+    asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(N_) : "memory");
+}
+#endif  // __HIPCC__
+
 }  // namespace tl
 
 #define TL_HIP_TRY(expr)                                                                        \

@@ -395,7 +395,7 @@ class HipDevice:
         _req(q, name="q"), _req(cache_k, name="cache_k"), _req(cache_v, name="cache_v")
         H, S, D = q.shape
         T = start_pos + S
-        ldv = (T + 31) // 32 * 32
+        ldv = (T + 63) // 64 * 64
         vT = self.empty(H, D, ldv)
         check(self.lib.tl_gather_vt_f16(_ptr(vT), _ptr(cache_v), T, ldv, H, D), "tl_gather_vt_f16")
         out = self.empty(S, H, D)

@@ -292,7 +292,7 @@ struct tlm_model {
             if (D == 64 || D == 128) {
                 // scores, scale, mask, softmax and the product with the values in one launch, keys read from the
                 // cache in place; only the values are transposed first                     Transformer.cpp:61-109
-                const int ldv = (T + 31) / 32 * 32;
+                const int ldv = (T + 63) / 64 * 64;
                 ck(tl_gather_vt_f16(values_c.p, cache_v[l].p, T, ldv, H, D), "gather_vt");
                 ck(tl_prefill_attention_f16(o_c.p, xq_c.p, cache_k[l].p, values_c.p, ldv, start_pos, S, H, D),
                    "prefill_attention");
@@ -392,7 +392,7 @@ int tlm_create(tlm_model** out, int dim, int hidden_dim, int n_layers, int n_hea
         m->scores.alloc(sc); m->scores2.alloc(sc); m->mask.alloc(sc);
         m->xq_c.alloc(sd); m->s_v.alloc(sd); m->o_c.alloc(sd);
         m->keys_c.alloc((size_t)max_seq_len * dim);
-        m->values_c.alloc((size_t)((max_seq_len + 31) / 32 * 32) * dim);   // rows padded for the prefill attention
+        m->values_c.alloc((size_t)((max_seq_len + 63) / 64 * 64) * dim);   // rows padded for the prefill attention
         m->logits.alloc(S * vocab_size);
         m->rope_table.alloc((size_t)max_seq_len * (dim / n_heads));
         ck(tl_rope_table_f16(m->rope_table.p, max_seq_len, dim / n_heads), "rope_table");

@@ -421,6 +421,31 @@ def test_prefill_attention(dev, oracle, H, S, D, start):
         assert np.array_equal(got[0].view(np.uint16), cv[0].view(np.uint16))
 
 
+@pytest.mark.parametrize("H,S,start", [(2, 1, 0), (3, 130, 0), (2, 257, 70), (33, 384, 0), (2, 640, 129), (20, 1000, 24),
+                                       (32, 2048, 0), (35, 1920, 37)])   # the last two: paired groups, even and odd count
+def test_prefill_attention_tiled_kernel(dev, oracle, H, S, start):
+    """The LDS-tiled kernel (workgroups of 128 query rows, key tiles of 64 staged once for four wavefronts; with many
+    groups a workgroup takes a long and a short one) does per wavefront what the one-wavefront kernel does: it is
+    checked against the CPU op chain where that is quick, and bit for bit against the other kernel everywhere."""
+    D, T = 128, start + S
+    q = synth.normal_f16(290, (H, S, D), 1.0)
+    ck = synth.normal_f16(291, (T, H, D), 1.0)
+    cv = synth.normal_f16(292, (T, H, D), 1.0)
+    qd, kd, vd = dev.from_numpy(q), dev.from_numpy(ck), dev.from_numpy(cv)
+    try:
+        dev.lib.tl_set_prefill_attention_variant(1)
+        one = dev.prefill_attention(qd, kd, vd, start).cpu().numpy()
+        dev.lib.tl_set_prefill_attention_variant(2)
+        tiled = dev.prefill_attention(qd, kd, vd, start).cpu().numpy()
+    finally:
+        dev.lib.tl_set_prefill_attention_variant(0)
+    assert np.array_equal(one.view(np.uint16), tiled.view(np.uint16))
+    if H * S * T <= 2 * 640 * 769:
+        assert_close_f16(tiled, oracle.attention_chain(q, ck, cv, start), RTOL, 3e-3, f"tiled prefill attention S={S} start={start}")
+    if start == 0:
+        assert np.array_equal(tiled[0].view(np.uint16), cv[0].view(np.uint16))
+
+
 def test_prefill_attention_limits(dev):
     from tensorlib_amd import TensorLibError
     with pytest.raises(TensorLibError):

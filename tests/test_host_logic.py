@@ -66,3 +66,49 @@ def test_no_gpu_means_loud_failure():
     from tensorlib_amd import HipDevice, TensorLibError
     with pytest.raises(TensorLibError):
         HipDevice(0)
+
+
+# ------------------------------------------------ arithmetic identities the kernels rely on ----
+
+def _round_to_f32(fr):
+    """Exact round-to-nearest-even of a Fraction to a float32 value (returned as Fraction)."""
+    from fractions import Fraction
+    if fr == 0:
+        return Fraction(0)
+    sign = -1 if fr < 0 else 1
+    a = abs(fr)
+    e = a.numerator.bit_length() - a.denominator.bit_length() - 24
+    while a / Fraction(2) ** e >= 2 ** 24:
+        e += 1
+    while a / Fraction(2) ** e < 2 ** 23:
+        e -= 1
+    e = max(e, -149)
+    scaled = a / Fraction(2) ** e
+    n = scaled.numerator // scaled.denominator
+    rem = scaled - n
+    if rem > Fraction(1, 2) or (rem == Fraction(1, 2) and n % 2 == 1):
+        n += 1
+    return sign * n * Fraction(2) ** e
+
+
+def test_score_quotient_by_newton_step_equals_the_division_for_every_half():
+    """The attention kernels form half(x / d) as q = x*r, q += fma(-q, d, x) * r with r = float32(1/d).  For every
+    finite fp16 x and both divisors in use (half(sqrt(64)) = 8, half(sqrt(128)) = 11.3125) this must round to the
+    same fp16 value as the fp32 division the reference performs (Transformer.cpp:94, half operator/)."""
+    from fractions import Fraction
+    for d_half in (np.float16(np.sqrt(64.0)), np.float16(np.sqrt(128.0))):
+        d = Fraction(float(d_half))
+        r = _round_to_f32(1 / d)
+        bits = np.arange(0, 0x7C00, dtype=np.uint16)            # non-negative finite halves; the scheme is odd in x
+        xs = bits.view(np.float16)
+        bad = []
+        for xv in xs:                                            # exact rational arithmetic, one rounding per operation
+            x = Fraction(float(xv))
+            q0 = _round_to_f32(x * r)
+            rem = _round_to_f32(x - q0 * d)
+            q1 = _round_to_f32(q0 + rem * r)
+            want32 = _round_to_f32(x / d)
+            got16, want16 = np.float16(np.float32(float(q1))), np.float16(np.float32(float(want32)))
+            if got16 != want16:
+                bad.append(float(xv))
+        assert not bad, (float(d_half), bad[:5])
