@@ -245,7 +245,8 @@ def bench_decode(dev, n_prompt: int = 128, n_generate: int = 256) -> dict:
     256 greedy steps, batch 1, max_seq 2048."""
     from . import synth
     cfg = Llama2Config()
-    m = Llama2Model(dev, cfg, max_tokens=n_prompt)
+    long_prompts = (512, 2048)
+    m = Llama2Model(dev, cfg, max_tokens=max(long_prompts))
     m.random_init_on_device(seed=7)
     prompt = synth.token_ids(11, n_prompt, cfg.vocab_size)
     res = {"config": "Llama2-7B fp16 random-init, prompt 128, 256 greedy steps, batch 1",
@@ -257,5 +258,18 @@ def bench_decode(dev, n_prompt: int = 128, n_generate: int = 256) -> dict:
         toks = (n_generate - 1) / td
         res[name] = {"decode_tok_s": round(toks, 2), "prefill_tok_s": round(n_prompt / tp, 1),
                      "frac_of_weight_streaming_ceiling": round(toks / ceiling, 4)}
+    # prefill of longer prompts (fused mode; logits of the last token only, as generate computes them)
+    import time
+    res["prefill_long"] = {}
+    for S in long_prompts:
+        ids = synth.token_ids(12, S, cfg.vocab_size)
+        m.forward(ids, 0, MODE_FUSED, all_logits=False)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        reps = 3
+        for _ in range(reps):
+            m.forward(ids, 0, MODE_FUSED, all_logits=False)
+        torch.cuda.synchronize()
+        res["prefill_long"][str(S)] = {"tok_s": round(S * reps / (time.perf_counter() - t0), 1)}
     m.close()
     return res
