@@ -48,11 +48,9 @@ constexpr int kPad = 8;  // halves of padding per LDS row
 // congruent mod 8 are dispatched to the same XCD) work on neighbouring tiles that share a
 // panel of B, and panels of B are walked once.
 __device__ __forceinline__ void tile_of_block(int bid, int nblocks, int tiles_m, int& tm, int& tn) {
-    int lid = bid;
-    if ((nblocks & 7) == 0) {
-        const int per_xcd = nblocks >> 3;
-        lid = (bid & 7) * per_xcd + (bid >> 3);
-    }
+    // XCD x takes a contiguous run of tiles: nblocks / 8 of them, one more on the first nblocks % 8 XCDs
+    const int x = bid & 7, base = nblocks >> 3, rem = nblocks & 7;
+    const int lid = x * base + (x < rem ? x : rem) + (bid >> 3);
     tm = lid % tiles_m;
     tn = lid / tiles_m;
 }
@@ -690,6 +688,7 @@ static int pick_variant(size_t M, size_t N, size_t K, int cus) {
     if (M <= 512 && tiles(256, 256) <= (size_t)cus) {
         const size_t enough = (size_t)cus * 6 / 10;
         if (tiles(256, 256) >= enough) return v_big;
+        if (M > 128 && tiles(128, 256) >= enough) return v_mid;   // measured ahead of 256x128 at equal tile counts
         if (M > 128 && tiles(256, 128) >= enough) return v_few_256x128;
         // a long K can be halved instead of narrowing the tile
         if (tiles(128, 128) >= enough || (K >= 8192 && tiles(128, 128) * 2 >= enough)) return v_few_128x128;
