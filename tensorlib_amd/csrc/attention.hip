@@ -481,7 +481,7 @@ prefill_attention_kernel(half_t* out, const half_t* q, const half_t* cache_k, co
 template <int D, bool PAIRED>
 __global__ void __launch_bounds__(256, 2)
 prefill_attention_tiled_kernel(half_t* out, const half_t* q, const half_t* cache_k, const half_t* vT, int ldv,
-                               int start_pos, int n_tokens, int n_heads, half_t divisor) {
+                               int start_pos, int n_tokens, int n_heads, half_t divisor, int slots) {
     static_assert(D == 128, "tile layout is written for head_dim 128");
     constexpr int KS = D / 16, DB = D / 32, TK = 64, NWQ = 4;
     constexpr int K_BYTES = TK * D * 2, V_BYTES = D * TK * 2, STAGE_BYTES = K_BYTES + V_BYTES;
@@ -492,7 +492,15 @@ prefill_attention_tiled_kernel(half_t* out, const half_t* q, const half_t* cache
 
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int h = blockIdx.y;
+    // One-dimensional grid of n_heads * slots workgroups (slots = query-group slots per head); ids congruent mod 8
+    // run on the same XCD, so XCD x takes a contiguous run of (head, slot) pairs and the workgroups that read one
+    // head's K and V share an L2.
+    const int nwg = (int)gridDim.x;
+    const int bid = (int)blockIdx.x;
+    const int xcd = bid & 7, per = nwg >> 3, rem = nwg & 7;
+    const int lid = xcd * per + (xcd < rem ? xcd : rem) + (bid >> 3);
+    const int h = lid / slots;
+    const int slot = lid % slots;
     const int T = start_pos + n_tokens;
     const int lr = lane & 31, lh = lane >> 5;
     const float dv = (float)divisor, rdv = 1.0f / dv;
@@ -534,9 +542,9 @@ prefill_attention_tiled_kernel(half_t* out, const half_t* q, const half_t* cache
     // tiles and the kernel does not end on a few long walks.
     const int n_groups = (n_tokens + 32 * NWQ - 1) / (32 * NWQ);
     for (int job = 0; job < 2; ++job) {
-        const int group = job == 0 ? n_groups - 1 - (int)blockIdx.x : (int)blockIdx.x;
+        const int group = job == 0 ? n_groups - 1 - slot : slot;
         if (job == 1) {
-            if (!PAIRED || group >= n_groups - 1 - (int)blockIdx.x) break;   // odd count: the middle group has no partner
+            if (!PAIRED || group >= n_groups - 1 - slot) break;   // odd count: the middle group has no partner
             asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");   // the stages are free again
         }
         const int qg0 = group * (32 * NWQ);                                    // first query row of the group
@@ -912,10 +920,12 @@ int tl_prefill_attention_f16(void* out, const void* q, const void* cache_k, cons
         const unsigned groups = (unsigned)((n_tokens + 127) / 128);
         // two workgroups fit a CU; beyond that a workgroup takes a long and a short group of 128 query rows
         const bool paired = (size_t)groups * (size_t)n_heads >= 2 * (size_t)tl::device_info().cu_count;
-        dim3 tgrid(paired ? (groups + 1) / 2 : groups, (unsigned)n_heads);
+        const unsigned slots = paired ? (groups + 1) / 2 : groups;   // workgroups per head
+        TL_REQUIRE((size_t)slots * (size_t)n_heads <= 0x7fffffffu, "tl_prefill_attention_f16: too many workgroups");
         auto kernel = paired ? tl::prefill_attention_tiled_kernel<128, true> : tl::prefill_attention_tiled_kernel<128, false>;
-        hipLaunchKernelGGL(kernel, tgrid, dim3(256), lds_bytes, tl::stream(), (tl::half_t*)out, (const tl::half_t*)q,
-                           (const tl::half_t*)cache_k, (const tl::half_t*)vT, ldv, start_pos, n_tokens, n_heads, divisor);
+        hipLaunchKernelGGL(kernel, dim3(slots * (unsigned)n_heads), dim3(256), lds_bytes, tl::stream(), (tl::half_t*)out,
+                           (const tl::half_t*)q, (const tl::half_t*)cache_k, (const tl::half_t*)vT, ldv, start_pos, n_tokens,
+                           n_heads, divisor, (int)slots);
         TL_CHECK_LAUNCH("prefill_attention_tiled_kernel");
         return TL_OK;
     }
