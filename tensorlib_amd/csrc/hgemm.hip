@@ -221,7 +221,7 @@ __global__ void __launch_bounds__(WM* WN * 64) hgemm_f16_dlds_kernel(HgemmArgs a
     // one (staged through the last stage's LDS), so the C stores and the cold start of the next tile overlap.
     // vmcnt counts loads and stores together on this ISA, so the stores are drained (vmcnt(0)) before the
     // next tile's loop resumes waiting with exact load counts.
-    constexpr bool PERSIST = (STAGES <= 3 && MODE == 1);
+    constexpr bool PERSIST = (STAGES <= 3 && MODE == 1 && NW * 32 * (BN / WN * 2 + 16) <= (BM + BN) * BK * 2);
 
     extern __shared__ __attribute__((aligned(1024))) unsigned char smem_raw[];
     typedef __attribute__((address_space(3))) unsigned char lds_byte_t;
@@ -492,7 +492,8 @@ __global__ void __launch_bounds__(WM* WN * 64) hgemm_f16_dlds_kernel(HgemmArgs a
         // whole 16-byte pieces of C rows (TN = 64: full 128-byte lines).  Rows are padded by 16 bytes so
         // that the 32 rows of one write land in different banks.
         constexpr int CH = TN / 8;               // 16-byte chunks per row
-        constexpr int RPR = 64 / CH;             // rows per wavefront-wide read
+        constexpr int RPR = 64 / CH;             // rows per wavefront-wide read (lanes beyond RPR * CH idle)
+        constexpr int PASSES = (32 + RPR - 1) / RPR;
         static_assert(NW * 32 * RS <= STAGES * STAGE_BYTES, "staging area must fit the ring");
         unsigned char* region = smem_raw + stage_area + wave * (32 * RS);
 #pragma unroll
@@ -506,8 +507,9 @@ __global__ void __launch_bounds__(WM* WN * 64) hgemm_f16_dlds_kernel(HgemmArgs a
                     *reinterpret_cast<half4_t*>(region + e_row * RS + (j * 32 + g * 8 + e_col) * 2) = h;
                 }
 #pragma unroll
-            for (int q = 0; q < 32 / RPR; ++q) {
+            for (int q = 0; q < PASSES; ++q) {
                 const int r = q * RPR + lane / CH, c = lane % CH;
+                if (lane >= RPR * CH || r >= 32) continue;
                 const half8_t v = *reinterpret_cast<const half8_t*>(region + r * RS + c * 16);
                 const int row = row_base + i * 32 + r, col = col_base + c * 8;
                 if (row < M && col < N) *reinterpret_cast<half8_t*>(C + (size_t)row * N + col) = v;
@@ -589,19 +591,21 @@ struct HgemmVariant {
     int bm, bn, bk, threads;
     int stages;  // 0: register-staged kernel (any K % 8 == 0); >= 2: direct-to-LDS ring (K % bk == 0)
     void (*kernel)(HgemmArgs);
+    bool persistent;  // the kernel walks tiles blockIdx.x, + gridDim.x, ... (same predicate as PERSIST in the kernel)
 };
 
 #define TL_HGEMM_VARIANT(BM, BN, BK, WM, WN) \
-    { "t" #BM "x" #BN "x" #BK "w" #WM "x" #WN, BM, BN, BK, WM * WN * 64, 0, hgemm_f16_mfma_kernel<BM, BN, BK, WM, WN> }
+    { "t" #BM "x" #BN "x" #BK "w" #WM "x" #WN, BM, BN, BK, WM * WN * 64, 0, hgemm_f16_mfma_kernel<BM, BN, BK, WM, WN>, false }
 #define TL_HGEMM_DLDS(BM, BN, BK, WM, WN, ST) \
     { "d" #BM "x" #BN "x" #BK "w" #WM "x" #WN "s" #ST, BM, BN, BK, WM * WN * 64, ST, \
-      hgemm_f16_dlds_kernel<BM, BN, BK, WM, WN, ST, 0> }
+      hgemm_f16_dlds_kernel<BM, BN, BK, WM, WN, ST, 0>, false }
 #define TL_HGEMM_PIPE(BM, BN, BK, WM, WN, ST) \
     { "p" #BM "x" #BN "x" #BK "w" #WM "x" #WN "s" #ST, BM, BN, BK, WM * WN * 64, ST, \
-      hgemm_f16_dlds_kernel<BM, BN, BK, WM, WN, ST, 1> }
+      hgemm_f16_dlds_kernel<BM, BN, BK, WM, WN, ST, 1>, \
+      (ST) <= 3 && (WM) * (WN) * 32 * ((BN) / (WN) * 2 + 16) <= ((BM) + (BN)) * (BK) * 2 }
 
 static const HgemmVariant g_variants[] = {
-    {"auto", 0, 0, 0, 0, 0, nullptr},
+    {"auto", 0, 0, 0, 0, 0, nullptr, false},
     // register-staged kernel: serves K % 64 != 0 (index 1 is the fallback of launch_hgemm)
     TL_HGEMM_VARIANT(128, 128, 64, 2, 2),  // 1
     TL_HGEMM_VARIANT(256, 256, 64, 2, 4),  // 2
@@ -621,6 +625,9 @@ static const HgemmVariant g_variants[] = {
     TL_HGEMM_PIPE(128, 128, 64, 2, 4, 4),  // 14
     TL_HGEMM_PIPE(128, 64, 64, 2, 2, 4),   // 15  few rows: narrow B tiles, deep ring
     TL_HGEMM_PIPE(128, 64, 64, 4, 1, 4),   // 16
+    // 192 columns: tile counts that fit 256 CUs where 128 and 256 columns do not (N = 11008, 12288)
+    TL_HGEMM_PIPE(128, 192, 64, 4, 2, 4),  // 17
+    TL_HGEMM_PIPE(256, 192, 64, 2, 2, 2),  // 18
 };
 
 static constexpr int kNumVariants = sizeof(g_variants) / sizeof(g_variants[0]);
@@ -674,8 +681,9 @@ static int hgemm_variant_index(const char* name) {
 // More rows: the tile shape with the cheapest schedule.  One round of 256x256 tiles on every CU costs R; a
 // round of 128x256 tiles (one workgroup per CU, three-stage ring: with B streamed from HBM a 0.6 us tile step
 // is shorter than the memory latency two stages can hide) does half the work in 0.61 R, a round of 128x128
-// tiles (two per CU) in 0.66 R, so the big tile wins unless its last round is mostly empty; a partly filled
-// round of a fraction f of the CUs costs about (0.65 + 0.3 f) of a full one (fewer busy CUs clock higher).
+// tiles (two per CU) in 0.66 R, a round of 256x192 tiles in 0.865 R, so the big tile wins unless its last round is
+// mostly empty; a partly filled round of a fraction f of the CUs costs about (0.65 + 0.3 f) of a full one (fewer
+// busy CUs clock higher).
 // Splitting K or peeling the last round off into a second K-split launch lost to this on every shape tried.
 static int pick_variant(size_t M, size_t N, size_t K, int cus) {
     static const int v_big = hgemm_variant_index("p256x256x64w2x4s2");
@@ -684,10 +692,14 @@ static int pick_variant(size_t M, size_t N, size_t K, int cus) {
     static const int v_few_256x128 = hgemm_variant_index("p256x128x64w2x4s3");
     static const int v_few_128x128 = hgemm_variant_index("p128x128x64w2x4s4");
     static const int v_few_128x64 = hgemm_variant_index("p128x64x64w4x1s4");
+    static const int v_few_128x192 = hgemm_variant_index("p128x192x64w4x2s4");
+    static const int v_256x192 = hgemm_variant_index("p256x192x64w2x2s2");
     auto tiles = [&](int bm, int bn) { return ((M + bm - 1) / bm) * ((N + bn - 1) / bn); };
     if (M <= 512 && tiles(256, 256) <= (size_t)cus) {
         const size_t enough = (size_t)cus * 6 / 10;
         if (tiles(256, 256) >= enough) return v_big;
+        // one round either way: 192 columns put more CUs to work than 256 (512x12288x4096: 58 vs 65 us)
+        if (M > 128 && tiles(128, 192) >= enough && tiles(128, 192) <= (size_t)cus) return v_few_128x192;
         if (M > 128 && tiles(128, 256) >= enough) return v_mid;   // measured ahead of 256x128 at equal tile counts
         if (M > 128 && tiles(256, 128) >= enough) return v_few_256x128;
         // a long K can be halved instead of narrowing the tile
@@ -703,8 +715,10 @@ static int pick_variant(size_t M, size_t N, size_t K, int cus) {
     const double c_big = cost(tiles(256, 256), (size_t)cus, 1.0);
     const double c_mid = cost(tiles(128, 256), (size_t)cus, 0.613);
     const double c_small = cost(tiles(128, 128), (size_t)cus * 2, 0.66);
+    const double c_192 = cost(tiles(256, 192), (size_t)cus, 0.865);   // three quarters of the work at 0.865 of the cost
     int best = v_big;
     double c = c_big;
+    if (c_192 < c * 0.97) { best = v_256x192; c = c_192; }
     if (c_mid < c * 0.97) { best = v_mid; c = c_mid; }
     if (c_small < c * 0.97) { best = v_small; c = c_small; }
     return best;
@@ -788,7 +802,7 @@ int launch_hgemm(const void* A, const void* B, void* C, size_t M, size_t N, size
     }
     // pipelined kernels with up to three stages are persistent: one workgroup per resident slot walks several tiles
     size_t grid_x = nblocks;
-    if (v.stages <= 3 && v.name[0] == 'p') {
+    if (v.persistent) {
         const size_t resident = (size_t)device_info().cu_count * ((160 * 1024) / lds > 0 ? (160 * 1024) / lds : 1);
         if (grid_x > resident) grid_x = resident;
     }
