@@ -20,12 +20,14 @@
  *   tlo_silu_f16, binary : float64 closed forms
  *   contiguous/set_item  : numpy as_strided
  *   argmax               : numpy argmax (first maximum)
- * PARITY UNPINNED (the reference cannot be compiled in the authoring container: it needs
- * cuda_fp16.h, and writing a stand-in header is not allowed): the *bit-exact* half-carried
- * chains tlo_softmax_f16_literal, tlo_rms_norm_f16_plain_literal and
- * tlo_silu_f16_cpu_literal.  They follow the reference text op by op but no golden vector
- * exists to confirm the last bit; they are only used to REPORT the distance between the
- * fp32-accumulating GPU kernels and the literal CPU half chain, never as a gate.
+ *   tlo_softmax_f16_literal, tlo_rms_norm_f16_plain_literal, tlo_silu_f16_cpu_literal (the half-carried
+ *                          chains of the literal CPU path): hand-worked consequences of half arithmetic: the
+ *                          running sum that stops at 2048 (softmax of n > 2048 equal values is 2^-11 each,
+ *                          RMSNorm of 4096 ones is 1.4140625), the shifted input rounded to half, the flipped
+ *                          sign of the half SiLU (x/(1+e^x) = -silu(-x), 0 far right, x far left).
+ * The reference itself cannot be compiled in the authoring container (it needs cuda_fp16.h, and writing a
+ * stand-in header is not allowed), so no vector produced by it exists; the literal chains are only used to
+ * REPORT the distance between the fp32-accumulating GPU kernels and the literal CPU half chain, never as a gate.
  */
 #include <math.h>
 #include <stddef.h>
@@ -207,7 +209,7 @@ void tlo_softmax_f16_f32(const h16* in, h16* out, size_t rows, size_t cols) {
 
 /* Literal half chain of softmaxImpl<half>, tensorLib/src/device/cpu/softmax.cpp:9-31:
  * half subtraction, exp rounded to half, sum carried in half, half division.
- * PARITY UNPINNED (see header). */
+ * Pinned by the saturating-sum and shifted-input cases of tests/test_oracle_pins.py. */
 void tlo_softmax_f16_literal(const h16* in, h16* out, size_t rows, size_t cols) {
 #pragma omp parallel for
     for (long i = 0; i < (long)rows; i++) {
@@ -263,7 +265,7 @@ void tlo_rms_norm_f16_exact(const h16* in, const h16* w, h16* out, float eps, in
 /* Literal CPU half chain of RMSNorm::forward_plain, tensorLib/src/nn/rmsNorm.cpp:14-56
  * through CPU<half> ops (pow: CPU.cpp:300-312; mean = sequential half sum then half
  * divide: CPU.cpp:340-354,389-395; scalar add; rsqrt: CPU.cpp:241-256; two half muls).
- * PARITY UNPINNED (see header). */
+ * Pinned by the saturating-mean cases of tests/test_oracle_pins.py. */
 void tlo_rms_norm_f16_plain_literal(const h16* in, const h16* w, h16* out, float eps, int hidden, int tokens) {
 #pragma omp parallel for
     for (int t = 0; t < tokens; t++) {
@@ -297,7 +299,8 @@ void tlo_silu_f16(const h16* in, h16* out, size_t n) {
 }
 
 /* Literal CPU half branch, tensorLib/src/device/cpu/CPU.cpp:216-219: the exponent has the
- * wrong sign (x * 1/(1+exp(+x))).  Kept only to document the deviation.  PARITY UNPINNED. */
+ * wrong sign (x * 1/(1+exp(+x))).  Kept only to document the deviation.
+ * Pinned by the identity -silu(-x) and its limits in tests/test_oracle_pins.py. */
 void tlo_silu_f16_cpu_literal(const h16* in, h16* out, size_t n) {
 #pragma omp parallel for
     for (long i = 0; i < (long)n; i++) {

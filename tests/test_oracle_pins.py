@@ -211,6 +211,33 @@ def test_softmax_literal_half_chain_is_close_but_not_the_gate(oracle):
     assert rel.max() > 1e-3          # ... but visibly less accurate than the fp32-sum form
 
 
+def test_softmax_literal_carries_its_sum_in_half(oracle):
+    """What the half arithmetic of softmax.cpp:20-24 fixes, worked by hand.  A row of n equal values: every
+    exponential is 1 and the running half sum counts 1, 2, ... exactly up to 2048; from there 2048 + 1 is a tie
+    that rounds to even, i.e. back to 2048, so for n > 2048 every output is 1/2048 = 2^-11 whatever n is, where a
+    float sum gives 1/n.  For n <= 2048 the outputs are half(1/n)."""
+    for n in (1, 3, 7, 100, 2048):
+        row = np.full((1, n), 0.75, np.float16)
+        assert np.all(oracle.softmax(row, literal=True) == np.float16(1.0 / n)), n
+    for n in (2049, 3000, 4096):
+        row = np.full((1, n), -3.0, np.float16)
+        assert np.all(oracle.softmax(row, literal=True) == np.float16(2.0 ** -11)), n
+        assert np.all(oracle.softmax(row) == np.float16(1.0 / n)), n        # the fp32-sum form, for contrast
+
+
+def test_softmax_literal_rounds_the_shifted_input_to_half(oracle):
+    """x - max is a half operation (softmax.cpp:20): 0.001 and 0.003 are different halves, but 10 away from the
+    row maximum both differences round to the same half, -10 (spacing 2^-7 there), so the literal chain gives
+    them the same probability, which a float subtraction does not."""
+    a, b = np.float16(0.001), np.float16(0.003)
+    assert a != b and np.float16(np.float32(a) - 10) == np.float16(np.float32(b) - 10)
+    row = np.array([[10.0, a, b]], np.float16)
+    lit = oracle.softmax(row, literal=True)[0]
+    assert lit[1] == lit[2] and lit[1] > 0
+    f32 = oracle.softmax(row)[0]
+    assert f32[1] != f32[2]
+
+
 # ---------------------------------------------------------------------------- RMSNorm ----
 
 def _rms_ref(x, w, eps):
@@ -252,6 +279,27 @@ def test_rms_norm_plain_literal_drifts(oracle):
     assert rel.max() < 1.0 and rel.mean() > 1e-2
 
 
+def test_rms_norm_plain_literal_saturating_mean(oracle):
+    """Hand-worked consequences of summing the squares sequentially in half (CPU.cpp:340-354): 4096 ones sum to
+    2048 (2048 + 1 ties back to 2048), so mean = 2048/4096 = 0.5, + half(1e-5) is still 0.5, rsqrt gives
+    half(1.41421) = 1.4140625 and every output is 1.4140625 where the definition gives 1.  With 2.0 the squares
+    are 4 and the sum stops at 8192 (8192 + 4 ties to even): mean 2, rsqrt half(0.70711) = 0.70703125, output
+    half(2 * 0.70703125) = 1.4140625 again.  Up to 2048 ones nothing saturates and the output is 1."""
+    w = np.ones(4096, np.float16)
+    out = oracle.rms_norm(np.ones((2, 4096), np.float16), w, 1e-5, "plain_literal")
+    assert np.all(out == np.float16(1.4140625))
+    out2 = oracle.rms_norm(np.full((1, 4096), 2.0, np.float16), w, 1e-5, "plain_literal")
+    assert np.all(out2 == np.float16(1.4140625))
+    out3 = oracle.rms_norm(np.ones((1, 2048), np.float16), np.ones(2048, np.float16), 1e-5, "plain_literal")
+    assert np.all(out3 == np.float16(1.0))
+    # the weight is applied after the normalisation, as a half multiply (rmsNorm.cpp:52-55)
+    w3 = np.full(4096, 3.0, np.float16)
+    out4 = oracle.rms_norm(np.ones((1, 4096), np.float16), w3, 1e-5, "plain_literal")
+    assert np.all(out4 == np.float16(np.float32(1.4140625) * 3))
+    # and for contrast the fp32-sum variant returns 1 on the same input
+    assert np.all(oracle.rms_norm(np.ones((1, 4096), np.float16), w, 1e-5, "fused") == np.float16(1.0))
+
+
 # ------------------------------------------------------------------------ elementwise ----
 
 def test_silu_closed_form(oracle):
@@ -268,6 +316,10 @@ def test_silu_cpu_literal_has_flipped_sign(oracle):
     lit = oracle.silu(x, cpu_literal=True).astype(np.float64)
     want = -oracle.silu((-x).astype(np.float16)).astype(np.float64)
     assert np.all(np.abs(lit - want) <= 2 * ulp16(want) + 1e-6)
+    # hand values: far right the half sigmoid 1/(1+e^x) underflows to 0 and the result is 0 where silu(x) = x;
+    # far left it is exactly 1 and the result is x where silu(x) = 0; at 0 it is 0 * 0.5
+    pts = np.array([20.0, 30.0, -20.0, -30.0, 0.0], np.float16)
+    assert np.array_equal(oracle.silu(pts, cpu_literal=True), np.array([0.0, 0.0, -20.0, -30.0, 0.0], np.float16))
 
 
 @pytest.mark.parametrize("op,fn", [("add", np.add), ("sub", np.subtract), ("mul", np.multiply), ("div", np.divide)])
