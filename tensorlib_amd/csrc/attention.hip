@@ -228,14 +228,36 @@ decode_attn_merge_kernel(half_t* out, const float* partial, int D, int n_chunks)
     const int d = threadIdx.x;
     if (d >= D) return;
     const float* base = partial + (size_t)h * n_chunks * (D + 2);
-    float m = -INFINITY;
-    for (int c = 0; c < n_chunks; ++c) m = fmaxf(m, base[(size_t)c * (D + 2)]);
-    float l = 0.f, o = 0.f;
-    for (int c = 0; c < n_chunks; ++c) {
-        const float* p = base + (size_t)c * (D + 2);
-        const float w = expf(p[0] - m);
-        l = __builtin_fmaf(p[1], w, l);
-        o = __builtin_fmaf(p[2 + d], w, o);
+    // Sixteen chunks per round trip (a long context has dozens of chunks, and a dependent load per chunk would
+    // cost a memory latency each), folded in with the online-softmax update, so the maxima need no pass of their
+    // own; the sums run over the chunks in ascending order.
+    constexpr int U = 16;
+    float m = -INFINITY, l = 0.f, o = 0.f;
+    for (int c0 = 0; c0 < n_chunks; c0 += U) {
+        float pm[U], pl[U], po[U];
+#pragma unroll
+        for (int j = 0; j < U; ++j) {
+            const float* p = base + (size_t)(c0 + j < n_chunks ? c0 + j : c0) * (D + 2);
+            pm[j] = p[0];
+            pl[j] = p[1];
+            po[j] = p[2 + d];
+        }
+        float m_new = m;
+#pragma unroll
+        for (int j = 0; j < U; ++j)
+            if (c0 + j < n_chunks) m_new = fmaxf(m_new, pm[j]);
+        const float scale = expf(m - m_new);   // 0 on the first round (m = -inf), 1 when the maximum stays
+        l *= scale;
+        o *= scale;
+        m = m_new;
+#pragma unroll
+        for (int j = 0; j < U; ++j) {
+            if (c0 + j < n_chunks) {
+                const float w = expf(pm[j] - m);
+                l = __builtin_fmaf(pl[j], w, l);
+                o = __builtin_fmaf(po[j], w, o);
+            }
+        }
     }
     out[(size_t)h * D + d] = (half_t)(o / l);
 }
