@@ -201,6 +201,14 @@ int tl_gemv_silu_mul_f16(const void* ab, const void* W, void* y, size_t N, size_
 int tl_gemv_add_rms_norm_f16(const void* x, const void* addend, const void* norm_weight, float eps,
                              const void* W, void* y, void* sum_out, size_t N, size_t K);
 
+/* sum_out[M,N] = residual + A[M,K] . W[N,K]^T and norm_out = rmsnorm(sum_out) * norm_weight: a Linear, the residual
+ * EwiseAdd and the RMSNorm that follow it in TransformerBlock::forward (model/llama2_7b/src/Transformer.cpp:165-175)
+ * for M token rows.  Same values as tl_matmul2d_f16 followed by tl_add_rms_norm_f16 (product rounded to fp16, sum
+ * rounded to fp16, fp32 mean of squares); when the GEMM splits K, its second pass is folded into the add + norm
+ * kernel.  norm_out also serves as the scratch for the product; it must not alias A or residual. */
+int tl_hgemm_add_rms_norm_f16(const void* A, const void* W, const void* residual, const void* norm_weight, float eps,
+                              void* sum_out, void* norm_out, size_t M, size_t N, size_t K);
+
 /* tl_rope_qk_store_kv_f16 + tl_decode_attention_f16 in one launch pair: qkv is the raw q|k|v
  * projection of the token at position `pos`; q is rotated on load, the rotated k and the v row
  * are written to cache_k[pos] / cache_v[pos], and out[h,:] attends to positions 0..pos.

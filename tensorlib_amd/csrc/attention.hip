@@ -725,10 +725,12 @@ add_rms_norm_kernel(half_t* sum_out, half_t* norm_out, const half_t* a, const ha
 
 // Same operation with every element held in registers between the two phases: one 16-byte load of
 // a, b and w per chunk, one global round trip in total.  512 threads, CPT chunks of 8 halves each.
-template <int CPT>
+// SLABS: b is not in memory yet: it is the result of a split-K GEMM whose fp32 slabs [splits][tokens][hidden] are
+// added here in split order and rounded to fp16, exactly what the GEMM's own second pass would have stored.
+template <int CPT, bool SLABS = false>
 __global__ void __launch_bounds__(512)
 add_rms_norm_vec_kernel(half_t* sum_out, half_t* norm_out, const half_t* a, const half_t* b, const half_t* w, float eps,
-                        int hidden) {
+                        int hidden, const float* slabs, int splits, size_t slab_stride) {
     __shared__ float red[8];
     const size_t base = (size_t)blockIdx.x * hidden;
     const int chunks = hidden / 8;
@@ -739,7 +741,25 @@ add_rms_norm_vec_kernel(half_t* sum_out, half_t* norm_out, const half_t* a, cons
         const int c = threadIdx.x + j * 512;
         const bool ok = c < chunks;
         va[j] = ok ? reinterpret_cast<const half8_t*>(a + base)[c] : zero8;
-        vb[j] = ok ? reinterpret_cast<const half8_t*>(b + base)[c] : zero8;
+        if constexpr (SLABS) {
+            vb[j] = zero8;
+            if (ok) {
+                const float4_t* p = reinterpret_cast<const float4_t*>(slabs + base) + 2 * c;
+                float4_t lo = p[0], hi = p[1];
+                for (int sp = 1; sp < splits; ++sp) {
+                    const float4_t* q = reinterpret_cast<const float4_t*>(slabs + (size_t)sp * slab_stride + base) + 2 * c;
+                    lo += q[0];
+                    hi += q[1];
+                }
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    vb[j][i] = (half_t)lo[i];
+                    vb[j][4 + i] = (half_t)hi[i];
+                }
+            }
+        } else {
+            vb[j] = ok ? reinterpret_cast<const half8_t*>(b + base)[c] : zero8;
+        }
         vw[j] = ok ? reinterpret_cast<const half8_t*>(w)[c] : zero8;
     }
     float ss = 0.f;
@@ -997,7 +1017,7 @@ int tl_add_rms_norm_f16(void* sum_out, void* norm_out, const void* a, const void
         auto launch = [&](auto kernel) {
             hipLaunchKernelGGL(kernel, dim3(num_tokens), dim3(512), 0, tl::stream(), (tl::half_t*)sum_out,
                                (tl::half_t*)norm_out, (const tl::half_t*)a, (const tl::half_t*)b,
-                               (const tl::half_t*)weight, eps, hidden_size);
+                               (const tl::half_t*)weight, eps, hidden_size, (const float*)nullptr, 0, (size_t)0);
         };
         if (cpt <= 1) launch(tl::add_rms_norm_vec_kernel<1>);
         else if (cpt == 2) launch(tl::add_rms_norm_vec_kernel<2>);
@@ -1008,6 +1028,34 @@ int tl_add_rms_norm_f16(void* sum_out, void* norm_out, const void* a, const void
                            (const tl::half_t*)weight, eps, hidden_size);
     }
     TL_CHECK_LAUNCH("add_rms_norm_kernel");
+    return TL_OK;
+}
+
+int tl_hgemm_add_rms_norm_f16(const void* A, const void* W, const void* residual, const void* norm_weight, float eps,
+                              void* sum_out, void* norm_out, size_t M, size_t N, size_t K) {
+    TL_ENSURE_INIT();
+    TL_REQUIRE(A && W && residual && norm_weight && sum_out && norm_out, "tl_hgemm_add_rms_norm_f16: null pointer");
+    TL_REQUIRE(N >= 1 && N <= 0x7fffffffu && M <= 0x7fffffffu, "tl_hgemm_add_rms_norm_f16: bad sizes");
+    if (M == 0) return TL_OK;
+    const bool vec = N % 8 == 0 && N <= 512 * 8 * 4 && tl::aligned16(sum_out) && tl::aligned16(norm_out) &&
+                     tl::aligned16(residual) && tl::aligned16(norm_weight);
+    float* slabs = nullptr;
+    int splits = 1;
+    // the product goes to norm_out (overwritten by the normalised rows afterwards) unless K was split
+    int rc = M == 1 ? tl::launch_gemv(A, W, norm_out, N, K, 1, 0, 0, 0, 0)
+                    : tl::launch_hgemm(A, W, norm_out, M, N, K, 1, 0, 0, 0, vec ? &slabs : nullptr, vec ? &splits : nullptr);
+    if (rc != TL_OK) return rc;
+    if (splits <= 1) return tl_add_rms_norm_f16(sum_out, norm_out, residual, norm_out, norm_weight, eps, (int)N, (int)M);
+    const int cpt = (int)((N / 8 + 511) / 512);
+    auto launch = [&](auto kernel) {
+        hipLaunchKernelGGL(kernel, dim3((unsigned)M), dim3(512), 0, tl::stream(), (tl::half_t*)sum_out, (tl::half_t*)norm_out,
+                           (const tl::half_t*)residual, (const tl::half_t*)nullptr, (const tl::half_t*)norm_weight, eps, (int)N,
+                           (const float*)slabs, splits, M * N);
+    };
+    if (cpt <= 1) launch(tl::add_rms_norm_vec_kernel<1, true>);
+    else if (cpt == 2) launch(tl::add_rms_norm_vec_kernel<2, true>);
+    else launch(tl::add_rms_norm_vec_kernel<4, true>);
+    TL_CHECK_LAUNCH("add_rms_norm_vec_kernel<slabs>");
     return TL_OK;
 }
 

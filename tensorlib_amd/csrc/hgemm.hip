@@ -725,7 +725,8 @@ static int pick_variant(size_t M, size_t N, size_t K, int cus) {
 }
 
 int launch_hgemm(const void* A, const void* B, void* C, size_t M, size_t N, size_t K, size_t batch, size_t sa,
-                 size_t sb, size_t sc) {
+                 size_t sb, size_t sc, float** partials_out, int* splits_out) {
+    if (splits_out) *splits_out = 1;
     if (M == 0 || N == 0 || batch == 0) return TL_OK;
     TL_REQUIRE(M <= 0x7fffffffu && N <= 0x7fffffffu && K <= 0x7fffffffu && batch <= 65535,
                "hgemm: size out of range");
@@ -821,6 +822,12 @@ int launch_hgemm(const void* A, const void* B, void* C, size_t M, size_t N, size
     }
     hipLaunchKernelGGL(v.kernel, dim3((unsigned)grid_x, (unsigned)batch, (unsigned)splits), dim3(v.threads), lds, st, a);
     TL_CHECK_LAUNCH(v.name);
+    if (splits > 1 && partials_out && splits_out) {
+        // the caller folds the second pass of split-K into its own kernel
+        *partials_out = a.partial;
+        *splits_out = splits;
+        return TL_OK;
+    }
     if (splits > 1) {
         const size_t n = M * N;
         size_t blocks = (n / 4 + 255) / 256;

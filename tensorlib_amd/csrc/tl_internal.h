@@ -51,8 +51,11 @@ struct GemvNormPrologue {
 };
 int launch_gemv(const void* x, const void* W, void* y, size_t N, size_t K, size_t batch, size_t sx,
                 size_t sw, size_t sy, int prologue, const GemvNormPrologue* norm = nullptr);
+// partials_out / splits_out (both or neither): when K was split, the fp32 slabs [splits][M][N] are handed to the
+// caller instead of being reduced into C (library-owned, valid until the next GEMM on the stream); *splits_out == 1
+// means C holds the result.
 int launch_hgemm(const void* A, const void* B, void* C, size_t M, size_t N, size_t K, size_t batch,
-                 size_t sa, size_t sb, size_t sc);
+                 size_t sa, size_t sb, size_t sc, float** partials_out = nullptr, int* splits_out = nullptr);
 
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 

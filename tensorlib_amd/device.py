@@ -316,6 +316,19 @@ class HipDevice:
         check(self.lib.tl_rope_qk_store_kv_f16(_ptr(qkv), _ptr(cache_k), _ptr(cache_v), pos, H, D),
               "tl_rope_qk_store_kv_f16")
 
+    def hgemm_add_rms_norm(self, A: torch.Tensor, W: torch.Tensor, residual: torch.Tensor, weight: torch.Tensor, eps: float):
+        """(residual + A . W^T, rmsnorm of that sum * weight) for [M, K] rows: a projection, the residual add and the
+        norm that follows it; a split-K GEMM's second pass happens inside the add + norm kernel."""
+        _req(A, name="A"), _req(W, name="W"), _req(residual, name="residual"), _req(weight, name="weight")
+        M, K = A.shape
+        N = W.shape[0]
+        if W.shape[1] != K or residual.shape != (M, N) or weight.numel() != N:
+            raise ValueError("shape mismatch")
+        s, n = self.empty(M, N), self.empty(M, N)
+        check(self.lib.tl_hgemm_add_rms_norm_f16(_ptr(A), _ptr(W), _ptr(residual), _ptr(weight), eps, _ptr(s), _ptr(n), M, N, K),
+              "tl_hgemm_add_rms_norm_f16")
+        return s, n
+
     def add_rms_norm(self, a: torch.Tensor, b: torch.Tensor, weight: torch.Tensor, eps: float, sum_out=None, norm_out=None):
         _req(a, name="a"), _req(b, name="b"), _req(weight, name="weight")
         hidden = a.shape[-1]

@@ -307,8 +307,9 @@ struct tlm_model {
                "scores.values");
             s_v.dev->contiguous(o_c.p, {1, S, H, D}, {H * S * D, D, S * D, 1}, 0, sd);
             }
-            matmul2d(o_c.p, w.wo, x_norm.p, S, dim, dim);
-            ck(tl_add_rms_norm_f16(x_residual.p, x_norm.p, x.p, x_norm.p, w.ffn_norm, eps, dim, S), "add_rms_norm");
+            // wo, h = x + attention, x_norm = rmsnorm(h) * ffn_norm (a split-K GEMM's second pass inside the norm kernel)
+            ck(tl_hgemm_add_rms_norm_f16(o_c.p, w.wo, x.p, w.ffn_norm, eps, x_residual.p, x_norm.p, S, dim, dim),
+               "hgemm_add_rms_norm");
             if (w.w3 == w.w1 + (size_t)hidden * dim && hidden % 8 == 0) {
                 matmul2d(x_norm.p, w.w1, x13.p, S, (size_t)2 * hidden, dim);   // rows of w1.x | w3.x
                 ck(tl_silu_mul_rows_f16(x2.p, x13.p, S, hidden), "silu_mul_rows");
@@ -317,9 +318,10 @@ struct tlm_model {
                 matmul2d(x_norm.p, w.w3, x3(S), S, hidden, dim);
                 ck(tl_silu_mul_f16(x2.p, x1(S), x3(S), (size_t)S * hidden), "silu_mul");
             }
-            matmul2d(x2.p, w.w2, x.p, S, dim, hidden);
+            // w2, x = h + ffn, x_norm = rmsnorm(x) * (next layer's attention norm | final norm)
             const half* next_norm = (l + 1 < n_layers) ? layers[l + 1].att_norm : final_norm;
-            ck(tl_add_rms_norm_f16(x.p, x_norm.p, x_residual.p, x.p, next_norm, eps, dim, S), "add_rms_norm");
+            ck(tl_hgemm_add_rms_norm_f16(x2.p, w.w2, x_residual.p, next_norm, eps, x.p, x_norm.p, S, dim, hidden),
+               "hgemm_add_rms_norm");
         }
     }
 

@@ -257,6 +257,28 @@ def test_decode_attention_rope_equals_separate_steps(dev, oracle, pos, H, D):
     assert_close_f16(got, _attention_chain_oracle(oracle, q_rot, ck, cv, pos + 1), RTOL, 2e-3, "fused rope attention")
 
 
+@pytest.mark.parametrize("M,N,K", [(128, 4096, 4096), (128, 4096, 11008), (512, 4096, 4096), (1, 4096, 4096), (37, 264, 328),
+                                   (128, 1000, 64), (2, 16384, 512)])
+def test_hgemm_add_rms_norm(dev, oracle, M, N, K):
+    """A projection, the residual add and the RMSNorm after it in one call: same bits as hgemm followed by
+    add_rms_norm whether or not the GEMM split K (then its second pass runs inside the norm kernel), and within
+    tolerance of the CPU chain."""
+    A = synth.normal_f16(150, (M, K), 1.0)
+    W = synth.normal_f16(151, (N, K), 0.02)
+    res = synth.normal_f16(152, (M, N), 1.0)
+    g = synth.normal_f16(153, (N,), 1.0)
+    Ad, Wd, rd, gd = dev.from_numpy(A), dev.from_numpy(W), dev.from_numpy(res), dev.from_numpy(g)
+    s_got, n_got = dev.hgemm_add_rms_norm(Ad, Wd, rd, gd, 1e-5)
+    y = dev.hgemm(Ad, Wd) if M > 1 else dev.gemv(Ad.view(-1), Wd).view(1, N)
+    s_want, n_want = dev.add_rms_norm(rd, y, gd, 1e-5)
+    assert np.array_equal(s_got.cpu().numpy().view(np.uint16), s_want.cpu().numpy().view(np.uint16))
+    assert np.array_equal(n_got.cpu().numpy().view(np.uint16), n_want.cpu().numpy().view(np.uint16))
+    if M * N * K <= 128 * 4096 * 4096:
+        s_cpu = oracle.binary(res, oracle.matmul2d(A, W), "add")
+        assert_close_scaled(s_got.cpu().numpy(), s_cpu, 1e-2, 1e-2, "hgemm + residual")
+        assert_close_scaled(n_got.cpu().numpy(), oracle.rms_norm(s_cpu, g, 1e-5, "fused"), 1e-2, 1e-2, "hgemm + residual + norm")
+
+
 @pytest.mark.parametrize("N,K", [(4096, 11008), (300, 512), (64, 4096), (33, 12288), (10, 520)])
 def test_gemv_silu_mul(dev, oracle, N, K):
     ab = synth.normal_f16(130, (2 * K,), 1.5)
