@@ -243,6 +243,13 @@ int tl_prefill_rope_qkv_f16(void* q_out, const void* q, const void* k, const voi
                             void* cache_k, void* cache_v, const void* rope_table, int start_pos, int n_tokens,
                             int n_heads, int head_dim);
 
+/* tl_prefill_rope_qkv_f16 for a fresh context (start_pos 0) that also writes the transposed value operand
+ * tl_gather_vt_f16 would build (vT[h][d][t] = v[t][h][d], zero for n_tokens <= t < ldv): one launch instead of two.
+ * head_dim 64 or 128, ldv a multiple of 64, row_stride a multiple of 8, 16-byte aligned pointers. */
+int tl_prefill_rope_qkv_vt_f16(void* q_out, const void* q, const void* k, const void* v, size_t row_stride, void* cache_k,
+                               void* cache_v, const void* rope_table, void* vT, int ldv, int n_tokens, int n_heads,
+                               int head_dim);
+
 /* vT[h][d][t] = cache_v[t][h][d] for t < T and 0 for T <= t < ldv (ldv % 8 == 0): the transposed value operand
  * of tl_prefill_attention_f16; the reference builds the same tensor with transpose + contiguous
  * (model/llama2_7b/src/Transformer.cpp:66-80). */

@@ -303,6 +303,45 @@ prefill_rope_qkv_kernel(half_t* q_out, const half_t* q, const half_t* k, const h
     *reinterpret_cast<half2_t*>(cache_v + c_off) = vv;
 }
 
+// prefill_rope_qkv_kernel and gather_vt_kernel in one pass for a fresh context (start_pos 0, so the new tokens are
+// all there is to transpose): workgroup (64-token tile, head), 16-byte accesses throughout; the tile of v goes
+// through LDS and leaves transposed, 128 contiguous bytes per head_dim row, zero beyond the last token.
+template <int D>
+__global__ void __launch_bounds__(256)
+prefill_rope_qkv_vt_kernel(half_t* q_out, const half_t* q, const half_t* k, const half_t* v, size_t ld, half_t* cache_k,
+                           half_t* cache_v, const half_t* rope_table, half_t* vT, int ldv, int n_tokens, int n_heads) {
+    constexpr int CH = D / 8;                     // 16-byte chunks per head row
+    __shared__ __attribute__((aligned(16))) half_t vt_tile[64][D + 8];
+    const int h = blockIdx.y;
+    const int s0 = blockIdx.x * 64;
+    const half8_t zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+    for (int it = threadIdx.x; it < 64 * CH; it += 256) {
+        const int sl = it / CH, c = it % CH;
+        const int s = s0 + sl;
+        half8_t vv = zero8;
+        if (s < n_tokens) {
+            const size_t in_off = (size_t)s * ld + (size_t)h * D + c * 8;
+            const half8_t cs = *reinterpret_cast<const half8_t*>(rope_table + ((size_t)s * (D / 2) + c * 4) * 2);
+            const half8_t qr = rope_chunk_cs(*reinterpret_cast<const half8_t*>(q + in_off), cs);
+            const half8_t kr = rope_chunk_cs(*reinterpret_cast<const half8_t*>(k + in_off), cs);
+            vv = *reinterpret_cast<const half8_t*>(v + in_off);
+            *reinterpret_cast<half8_t*>(q_out + ((size_t)h * n_tokens + s) * D + c * 8) = qr;
+            const size_t c_off = ((size_t)s * n_heads + h) * D + c * 8;
+            *reinterpret_cast<half8_t*>(cache_k + c_off) = kr;
+            *reinterpret_cast<half8_t*>(cache_v + c_off) = vv;
+        }
+        *reinterpret_cast<half8_t*>(&vt_tile[sl][c * 8]) = vv;
+    }
+    __syncthreads();
+    for (int it = threadIdx.x; it < D * 8; it += 256) {
+        const int d = it / 8, j = it % 8;
+        half8_t o;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) o[i] = vt_tile[8 * j + i][d];
+        *reinterpret_cast<half8_t*>(vT + ((size_t)h * D + d) * ldv + s0 + 8 * j) = o;
+    }
+}
+
 // vT[h][d][t] = cache_v[t][h][d] for t < T, zero for T <= t < ldv: the value operand of the prefill attention,
 // rows of `ldv` elements (a multiple of 8, so that groups of four positions can be read with 8-byte loads).
 __global__ void __launch_bounds__(256)
@@ -917,6 +956,31 @@ int tl_prefill_rope_qkv_f16(void* q_out, const void* q, const void* k, const voi
                        (tl::half_t*)cache_k, (tl::half_t*)cache_v, (const tl::half_t*)rope_table, start_pos, n_tokens,
                        n_heads, head_dim);
     TL_CHECK_LAUNCH("prefill_rope_qkv_kernel");
+    return TL_OK;
+}
+
+int tl_prefill_rope_qkv_vt_f16(void* q_out, const void* q, const void* k, const void* v, size_t row_stride, void* cache_k,
+                               void* cache_v, const void* rope_table, void* vT, int ldv, int n_tokens, int n_heads,
+                               int head_dim) {
+    TL_ENSURE_INIT();
+    TL_REQUIRE(q_out && q && k && v && cache_k && cache_v && rope_table && vT, "tl_prefill_rope_qkv_vt_f16: null pointer");
+    TL_REQUIRE(n_tokens >= 1 && n_heads >= 1 && n_heads <= 65535, "tl_prefill_rope_qkv_vt_f16: bad sizes");
+    TL_REQUIRE(head_dim == 64 || head_dim == 128, "tl_prefill_rope_qkv_vt_f16: head_dim %d not supported (64 or 128)", head_dim);
+    TL_REQUIRE(ldv % 64 == 0 && ldv >= n_tokens, "tl_prefill_rope_qkv_vt_f16: ldv=%d must be a multiple of 64 that covers the tokens", ldv);
+    TL_REQUIRE(row_stride % 8 == 0 && row_stride >= (size_t)n_heads * head_dim,
+               "tl_prefill_rope_qkv_vt_f16: row stride %zu too small or not a multiple of 8", row_stride);
+    TL_REQUIRE(tl::aligned16(q_out) && tl::aligned16(q) && tl::aligned16(k) && tl::aligned16(v) && tl::aligned16(cache_k) &&
+                   tl::aligned16(cache_v) && tl::aligned16(rope_table) && tl::aligned16(vT),
+               "tl_prefill_rope_qkv_vt_f16: pointers must be 16-byte aligned");
+    dim3 grid((unsigned)(ldv / 64), (unsigned)n_heads);
+    auto launch = [&](auto kernel) {
+        hipLaunchKernelGGL(kernel, grid, dim3(256), 0, tl::stream(), (tl::half_t*)q_out, (const tl::half_t*)q,
+                           (const tl::half_t*)k, (const tl::half_t*)v, row_stride, (tl::half_t*)cache_k, (tl::half_t*)cache_v,
+                           (const tl::half_t*)rope_table, (tl::half_t*)vT, ldv, n_tokens, n_heads);
+    };
+    if (head_dim == 64) launch(tl::prefill_rope_qkv_vt_kernel<64>);
+    else launch(tl::prefill_rope_qkv_vt_kernel<128>);
+    TL_CHECK_LAUNCH("prefill_rope_qkv_vt_kernel");
     return TL_OK;
 }
 

@@ -384,6 +384,26 @@ class HipDevice:
               "tl_prefill_rope_qkv_f16")
         return out
 
+
+    def prefill_rope_qkv_vt(self, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, cache_k: torch.Tensor,
+                            cache_v: torch.Tensor, table: torch.Tensor, n_heads: int):
+        """prefill_rope_qkv at start_pos 0 that also returns the transposed value operand of prefill_attention
+        ([n_heads, head_dim, ldv], ldv = tokens rounded up to 64, zero padded)."""
+        for t, nm in ((q, "q"), (k, "k"), (v, "v")):
+            if t.dtype != torch.float16 or not t.is_cuda or t.dim() != 2 or t.stride(1) != 1:
+                raise ValueError(f"{nm} must be a 2-D fp16 device tensor with unit column stride")
+        S, dim = q.shape
+        ld = q.stride(0)
+        if k.stride(0) != ld or v.stride(0) != ld or k.shape != q.shape or v.shape != q.shape:
+            raise ValueError("q, k, v must share shape and row stride")
+        D = dim // n_heads
+        ldv = (S + 63) // 64 * 64
+        out = torch.empty((n_heads, S, D), dtype=torch.float16, device=q.device)
+        vT = torch.empty((n_heads, D, ldv), dtype=torch.float16, device=q.device)
+        check(self.lib.tl_prefill_rope_qkv_vt_f16(_ptr(out), q.data_ptr(), k.data_ptr(), v.data_ptr(), ld, _ptr(cache_k),
+                                                  _ptr(cache_v), _ptr(table), _ptr(vT), ldv, S, n_heads, D),
+              "tl_prefill_rope_qkv_vt_f16")
+        return out, vT
     def scaled_causal_softmax(self, scores: torch.Tensor, divisor: float, start_pos: int) -> torch.Tensor:
         """In place on scores [n_heads, S, start_pos + S]: divide by half(divisor), causal mask, softmax."""
         _req(scores, name="scores")

@@ -287,13 +287,20 @@ struct tlm_model {
                 matmul2d(x_norm.p, w.wv, xv(S), S, dim, dim);
                 q = xq(S); k = xk(S); v = xv(S); ld = dim;
             }
-            ck(tl_prefill_rope_qkv_f16(xq_c.p, q, k, v, ld, cache_k[l].p, cache_v[l].p, rope_table.p, start_pos, S, H, D),
-               "prefill_rope_qkv");
+            const int ldv = (T + 63) / 64 * 64;
+            const bool one_pass = (D == 64 || D == 128) && start_pos == 0 && ld % 8 == 0;
+            if (one_pass) {
+                // a fresh context: the transposed values are written along with the rotated q, k and the cache rows
+                ck(tl_prefill_rope_qkv_vt_f16(xq_c.p, q, k, v, ld, cache_k[l].p, cache_v[l].p, rope_table.p, values_c.p, ldv,
+                                              S, H, D), "prefill_rope_qkv_vt");
+            } else {
+                ck(tl_prefill_rope_qkv_f16(xq_c.p, q, k, v, ld, cache_k[l].p, cache_v[l].p, rope_table.p, start_pos, S, H, D),
+                   "prefill_rope_qkv");
+            }
             if (D == 64 || D == 128) {
                 // scores, scale, mask, softmax and the product with the values in one launch, keys read from the
                 // cache in place; only the values are transposed first                     Transformer.cpp:61-109
-                const int ldv = (T + 63) / 64 * 64;
-                ck(tl_gather_vt_f16(values_c.p, cache_v[l].p, T, ldv, H, D), "gather_vt");
+                if (!one_pass) ck(tl_gather_vt_f16(values_c.p, cache_v[l].p, T, ldv, H, D), "gather_vt");
                 ck(tl_prefill_attention_f16(o_c.p, xq_c.p, cache_k[l].p, values_c.p, ldv, start_pos, S, H, D),
                    "prefill_attention");
             } else {

@@ -396,6 +396,36 @@ def test_prefill_rope_qkv(dev, oracle, S, H, D, start, fused_rows):
     assert np.array_equal(got_q.view(np.uint16), two.view(np.uint16))
 
 
+@pytest.mark.parametrize("S,H,D,fused_rows", [(128, 32, 128, True), (70, 3, 128, True), (1, 2, 64, False), (200, 5, 64, True),
+                                              (64, 4, 128, False)])
+def test_prefill_rope_qkv_vt_equals_the_two_launches(dev, S, H, D, fused_rows):
+    """The one-pass kernel for a fresh context against prefill_rope_qkv followed by gather_vt: rotated q, both
+    cache rows and the transposed, zero-padded values, bit for bit (the pair is checked against the CPU above)."""
+    dim = H * D
+    qkv = synth.normal_f16(170, (S, 3 * dim), 1.0)
+    ck0 = synth.normal_f16(171, (S + 2, H, D), 1.0)
+    cv0 = synth.normal_f16(172, (S + 2, H, D), 1.0)
+    table = dev.rope_table(S + 2, D)
+
+    def inputs():
+        if fused_rows:
+            t = dev.from_numpy(qkv)
+            return t[:, :dim], t[:, dim:2 * dim], t[:, 2 * dim:]
+        return tuple(dev.from_numpy(np.ascontiguousarray(qkv[:, i * dim:(i + 1) * dim])) for i in range(3))
+
+    k1, v1 = dev.from_numpy(ck0), dev.from_numpy(cv0)
+    q1 = dev.prefill_rope_qkv(*inputs(), k1, v1, table, 0, H)
+    ldv = (S + 63) // 64 * 64
+    vT1 = dev.empty(H, D, ldv)
+    from tensorlib_amd._lib import check
+    check(dev.lib.tl_gather_vt_f16(vT1.data_ptr(), v1.data_ptr(), S, ldv, H, D), "tl_gather_vt_f16")
+    k2, v2 = dev.from_numpy(ck0), dev.from_numpy(cv0)
+    q2, vT2 = dev.prefill_rope_qkv_vt(*inputs(), k2, v2, table, H)
+    assert torch.equal(q1, q2) and torch.equal(k1, k2) and torch.equal(v1, v2)
+    assert torch.equal(vT1, vT2)
+    assert vT2.shape[2] == ldv and (ldv == S or bool((vT2[:, :, S:] == 0).all()))
+
+
 @pytest.mark.parametrize("H,S,start", [(32, 128, 0), (4, 17, 9), (2, 1, 300), (3, 70, 0)])
 def test_scaled_causal_softmax(dev, oracle, H, S, start):
     """ScalarDiv, mask add and softmax of Attention::forward in one launch, against the three CPU ops."""
