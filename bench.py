@@ -42,7 +42,7 @@ HGEMM_SHAPES = [(2048, 4096, 4096), (2048, 11008, 4096), (2048, 32000, 4096), (2
 # HBM bytes per GEMV launch measured with rocprofv3 --pmc (FETCH_SIZE, WRITE_SIZE), averaged over
 # the four sweep launches and scaled by the same counters' reading for a copy kernel of known
 # size (FETCH_SIZE x 1.9997 KiB, WRITE_SIZE x 1.0000 KiB); algorithmic bytes per launch are 119,050,624.
-GEMV_TRAFFIC_BYTES_PER_LAUNCH = 119_424_897  # profiles/gemv_decode_sweep_hbm_traffic.txt
+GEMV_TRAFFIC_BYTES_PER_LAUNCH = 119_423_152  # profiles/gemv_decode_sweep_hbm_traffic.txt
 
 
 def parse_args():
