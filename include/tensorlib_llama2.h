@@ -88,6 +88,27 @@ int tlm_forward(tlm_model* m, const int* dev_tokens, int n_tokens, int start_pos
 int tlm_generate(tlm_model* m, const int* host_prompt, int n_prompt, int n_generate, int mode,
                  int* host_out_tokens, double* prefill_seconds, double* decode_seconds);
 
+/* Llama2::text_completion and one turn of Llama2::chat (model/llama2_7b/src/llama2.cpp:103-107,120-148) on
+ * top of Llama2::generate (llama2.cpp:15-101), with the tokenizer of include/tensorlib_tokenizer.h.
+ *   chat_template != 0 renders "[INST] <text> [/INST]" first (llama2.cpp:131,137);
+ *   the text is encoded with BOS and without EOS (llama2.cpp:105,143) and must fit max_tokens;
+ *   *position is the reference's process-wide `total_len` (llama2.cpp:13), owned by the caller here: the prompt
+ *   is prefilled at [*position, *position + n_prompt), and *position advances by the prompt length plus the
+ *   number of decode steps run (llama2.cpp:52,83), so the next turn continues in the same KV cache;
+ *   the token picked from the prefill logits is always emitted (llama2.cpp:57-63); each of the up to
+ *   n_generate decode steps (the reference runs 256) picks the next token and stops, without emitting it, on
+ *   BOS (1) or EOS (2) (llama2.cpp:88-91);
+ *   every emitted token goes to on_piece (may be NULL) with its piece decoded as the reference prints it,
+ *   tokenizer.decode(-1, token) (llama2.cpp:63,93); the bytes are not terminated and only valid during the call.
+ * *n_decode_steps receives the number of decode steps run (the reference's generate_cnt).  The host reads one
+ * token id per step, as the reference does (llama2.cpp:85); benchmarks use tlm_generate, which does not.
+ * Declared with an opaque tokenizer pointer so this header does not depend on the tokenizer's. */
+struct tlt_tokenizer;
+typedef void (*tlm_piece_fn)(const char* bytes, size_t n_bytes, int token, void* user);
+int tlm_text_completion(tlm_model* m, const struct tlt_tokenizer* tok, const char* text, int chat_template,
+                        int* position, int n_generate, int mode, tlm_piece_fn on_piece, void* user,
+                        int* n_decode_steps, double* prefill_seconds, double* decode_seconds);
+
 int tlm_get_buffer(tlm_model* m, int which, int layer, void** dev_ptr);
 
 #ifdef __cplusplus

@@ -22,6 +22,7 @@
 
 #include "tensorlib_amd.h"
 #include "tensorlib_llama2.h"
+#include "tensorlib_tokenizer.h"
 #include "tl_hip_device.hpp"
 
 namespace {
@@ -596,6 +597,69 @@ int tlm_generate(tlm_model* m, const int* host_prompt, int n_prompt, int n_gener
         if (decode_seconds) *decode_seconds = std::chrono::duration<double>(t2 - t1).count();
     } catch (const std::exception& e) {
         return fail("tlm_generate: %s", e.what());
+    }
+    return 0;
+}
+
+int tlm_text_completion(tlm_model* m, const tlt_tokenizer* tok, const char* text, int chat_template, int* position,
+                        int n_generate, int mode, tlm_piece_fn on_piece, void* user, int* n_decode_steps,
+                        double* prefill_seconds, double* decode_seconds) {
+    if (!m || !tok || !text || !position) return fail("tlm_text_completion: null argument");
+    if (*position < 0 || n_generate < 0) return fail("tlm_text_completion: negative position or step count");
+    using clock = std::chrono::steady_clock;
+    try {
+        std::string prompt = chat_template ? "[INST] " + std::string(text) + " [/INST]" : std::string(text);
+        std::vector<int> ids(prompt.size() + 2);
+        size_t n_ids = 0;
+        if (tlt_encode(tok, prompt.data(), prompt.size(), 1, 0, ids.data(), ids.size(), &n_ids) != 0)
+            return fail("tlm_text_completion: %s", tlt_last_error());
+        const int n_prompt = (int)n_ids, start = *position;
+        if (n_prompt < 1 || n_prompt > m->max_tokens)
+            return fail("tlm_text_completion: prompt of %d tokens not in [1,%d]", n_prompt, m->max_tokens);
+        // room for the prompt, the token picked after it and one token per decode step
+        const long last = (long)start + n_prompt + n_generate;
+        if (last > m->max_seq || last + 1 > m->d_tokens_cap)
+            return fail("tlm_text_completion: position %d + %d prompt tokens + %d steps exceeds max_seq_len %d", start,
+                        n_prompt, n_generate, m->max_seq);
+        std::vector<char> piece(256);
+        auto emit = [&](int token) {
+            if (!on_piece) return;
+            size_t nb = 0;
+            if (tlt_decode(tok, -1, token, piece.data(), piece.size(), &nb) != 0) {
+                piece.resize(1 << 16);
+                if (tlt_decode(tok, -1, token, piece.data(), piece.size(), &nb) != 0)
+                    throw std::runtime_error(tlt_last_error());
+            }
+            on_piece(piece.data(), nb, token, user);
+        };
+        // d_tokens[i] is the token at position i, as in tlm_generate
+        ck(tl_memcpy_h2d(m->d_tokens + start, ids.data(), (size_t)n_prompt * sizeof(int)), "prompt h2d");
+        ck(tl_synchronize(), "sync");
+        auto t0 = clock::now();
+        int pos = start + n_prompt;  // position of the token picked next
+        half* lg = m->forward(m->d_tokens + start, n_prompt, start, mode, false);
+        ck(tl_argmax_f16(m->d_tokens + pos, lg, m->vocab, m->vocab), "argmax");
+        int token = 0;
+        ck(tl_memcpy_d2h(&token, m->d_tokens + pos, sizeof(int)), "token d2h");
+        auto t1 = clock::now();
+        emit(token);
+        int steps = 0;
+        while (steps < n_generate) {
+            lg = m->forward(m->d_tokens + pos, 1, pos, mode, false);
+            ck(tl_argmax_f16(m->d_tokens + pos + 1, lg, m->vocab, m->vocab), "argmax");
+            ++pos;
+            ++steps;
+            ck(tl_memcpy_d2h(&token, m->d_tokens + pos, sizeof(int)), "token d2h");
+            if (token == 1 || token == 2) break;
+            emit(token);
+        }
+        auto t2 = clock::now();
+        *position = pos;
+        if (n_decode_steps) *n_decode_steps = steps;
+        if (prefill_seconds) *prefill_seconds = std::chrono::duration<double>(t1 - t0).count();
+        if (decode_seconds) *decode_seconds = std::chrono::duration<double>(t2 - t1).count();
+    } catch (const std::exception& e) {
+        return fail("tlm_text_completion: %s", e.what());
     }
     return 0;
 }

@@ -25,10 +25,13 @@ _PROTOS = {
     "tlm_set_weight": (_i, [_vp, _i, _i, _vp]),
     "tlm_forward": (_i, [_vp, _vp, _i, _i, _i, _i, ctypes.POINTER(_vp)]),
     "tlm_generate": (_i, [_vp, _vp, _i, _i, _i, _vp, ctypes.POINTER(ctypes.c_double), ctypes.POINTER(ctypes.c_double)]),
+    "tlm_text_completion": (_i, [_vp, _vp, ctypes.c_char_p, _i, ctypes.POINTER(_i), _i, _i, _vp, _vp, ctypes.POINTER(_i),
+                                 ctypes.POINTER(ctypes.c_double), ctypes.POINTER(ctypes.c_double)]),
     "tlm_get_buffer": (_i, [_vp, _i, _i, ctypes.POINTER(_vp)]),
     "tlm_load_checkpoint": (_i, [ctypes.c_char_p, _i, _i, ctypes.POINTER(_vp)]),
     "tlm_get_config": (_i, [_vp, ctypes.POINTER(_i)]),
 }
+_PIECE_FN = ctypes.CFUNCTYPE(None, ctypes.POINTER(ctypes.c_char), ctypes.c_size_t, _i, _vp)
 _llib = None
 
 
@@ -238,6 +241,30 @@ class Llama2Model:
         _ck(self.l.tlm_generate(self.h, prompt.ctypes.data_as(_vp), prompt.size, n_generate, mode,
                                 out.ctypes.data_as(_vp), ctypes.byref(tp), ctypes.byref(td)), "tlm_generate")
         return out, tp.value, td.value
+
+
+    def text_completion(self, tokenizer, text, position: int = 0, n_generate: int = 256, mode: int = MODE_FUSED,
+                        chat_template: bool = False, on_piece=None):
+        """Llama2::text_completion, or one chat turn with chat_template=True (model/llama2_7b/src/llama2.cpp:103-148).
+        Returns (emitted token ids, their text as bytes, new position, decode steps run, prefill s, decode s);
+        on_piece(bytes, token) is called as each token is produced."""
+        raw = text.encode("utf-8") if isinstance(text, str) else bytes(text)
+        tokens, chunks = [], []
+
+        def _piece(ptr, n, token, _user):
+            b = ctypes.string_at(ptr, n)
+            tokens.append(int(token))
+            chunks.append(b)
+            if on_piece is not None:
+                on_piece(b, int(token))
+
+        cb = _PIECE_FN(_piece)
+        pos, steps = _i(position), _i(0)
+        tp, td = ctypes.c_double(), ctypes.c_double()
+        _ck(self.l.tlm_text_completion(self.h, tokenizer.h, raw, int(chat_template), ctypes.byref(pos), n_generate, mode,
+                                       ctypes.cast(cb, _vp), None, ctypes.byref(steps), ctypes.byref(tp),
+                                       ctypes.byref(td)), "tlm_text_completion")
+        return tokens, b"".join(chunks), pos.value, steps.value, tp.value, td.value
 
 
 def bench_decode(dev, n_prompt: int = 128, n_generate: int = 256) -> dict:

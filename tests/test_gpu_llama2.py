@@ -76,6 +76,81 @@ def test_toy_model_generate_matches_stepwise_forward(dev):
     m.close(), m2.close()
 
 
+def _toy_tokenizer(tmp_path):
+    from tensorlib_amd.tokenizer import Tokenizer, write_tokenizer_file
+    pieces = [b"<unk>", b"\n<s>\n", b"\n</s>\n"] + [f"<0x{b:02X}>".encode() for b in range(256)]
+    scores = [0.0] * len(pieces)
+    for i, (p, sc) in enumerate([(b" ", -1.0), (b"a", -2.0), (b"b", -3.0), (b"c", -4.0), (b"ab", -0.5), (b" a", -0.7),
+                                 (b" ab", -0.2), (b"abc", -0.9), (b"bc", -0.1), (b"[", -3.5), (b"]", -3.6),
+                                 (b"INST", -0.3), (b"/", -3.7), (b" [", -0.8), (b"[INST]", -0.05)]):
+        pieces.append(p)
+        scores.append(sc)
+    path = str(tmp_path / "tok.bin")
+    write_tokenizer_file(path, pieces, scores)
+    return Tokenizer(path, len(pieces))
+
+
+def _stepwise_completion(dev, model, tok, text, position, n_generate, mode):
+    """The reference's generate loop (model/llama2_7b/src/llama2.cpp:51-95) spelled out with tlm_forward, a device
+    argmax read back per step and the tokenizer's decode(-1, token)."""
+    prompt = tok.encode(text, bos=True, eos=False)
+    lg = model.forward(prompt, position, mode, all_logits=False)
+    position += len(prompt)
+    t = int(dev.argmax(lg)[0].item())
+    emitted, steps = [t], 0
+    for _ in range(n_generate):
+        lg = model.forward([t], position, mode)
+        position += 1
+        steps += 1
+        t = int(dev.argmax(lg)[0].item())
+        if t in (1, 2):
+            break
+        emitted.append(t)
+    return emitted, b"".join(tok.decode_piece(-1, x) for x in emitted), position, steps
+
+
+def test_text_completion_and_chat_turns_follow_the_reference_loop(dev, tmp_path):
+    """tlm_text_completion: prompt encoding with BOS, streaming of decode(-1, token), a second turn that goes on
+    at the carried position with the chat template, and the stop on EOS without emitting it."""
+    from tensorlib_amd import TensorLibError
+    from tensorlib_amd.llama2 import MODE_FUSED, MODE_REFERENCE_CHAIN, Llama2Config, Llama2Model
+    tok = _toy_tokenizer(tmp_path)
+    cfg = Llama2Config(dim=256, hidden_dim=688, n_layers=2, n_heads=4, vocab_size=tok.vocab_size, max_seq_len=96)
+    w = _weights(cfg, 4000)
+    w["classifier"][1:3] = 0            # BOS / EOS never win in the first part
+    for mode in (MODE_FUSED, MODE_REFERENCE_CHAIN):
+        m, m2 = Llama2Model(dev, cfg, max_tokens=32), Llama2Model(dev, cfg, max_tokens=32)
+        m.set_weights(w), m2.set_weights(w)
+        streamed = []
+        toks, text, pos, steps, tp, td = m.text_completion(tok, "ab c abc", 0, 12, mode,
+                                                           on_piece=lambda b, t: streamed.append((b, t)))
+        want = _stepwise_completion(dev, m2, tok, "ab c abc", 0, 12, mode)
+        assert (toks, text, pos, steps) == want
+        assert steps == 12 and len(toks) == 13 and pos == len(tok.encode("ab c abc")) + 12
+        assert [t for _, t in streamed] == toks and b"".join(b for b, _ in streamed) == text
+        assert tp > 0 and td > 0
+        # second turn: chat template, continues in the same KV cache at the carried position
+        toks2, text2, pos2, steps2, _, _ = m.text_completion(tok, "bc a", pos, 9, mode, chat_template=True)
+        want2 = _stepwise_completion(dev, m2, tok, "[INST] bc a [/INST]", pos, 9, mode)
+        assert (toks2, text2, pos2, steps2) == want2
+        with pytest.raises(TensorLibError):     # would run past max_seq_len
+            m.text_completion(tok, "a", pos2, 96, mode)
+        m.close(), m2.close()
+    # stop on EOS: let EOS win exactly where the free run picked the first token it had not picked before
+    k = next((i for i in range(1, len(toks)) if toks[i] not in toks[:i]), None)
+    assert k is not None, f"degenerate toy run {toks}"
+    w_stop = dict(w)
+    w_stop["classifier"] = w["classifier"].copy()
+    w_stop["classifier"][2] = w["classifier"][toks[k]]
+    w_stop["classifier"][toks[k]] = 0
+    m = Llama2Model(dev, cfg, max_tokens=32)
+    m.set_weights(w_stop)
+    toks3, text3, pos3, steps3, _, _ = m.text_completion(tok, "ab c abc", 0, 12, MODE_REFERENCE_CHAIN)
+    assert toks3 == toks[:k] and steps3 == k and pos3 == len(tok.encode("ab c abc")) + k
+    assert text3 == b"".join(tok.decode_piece(-1, x) for x in toks[:k])
+    m.close()
+
+
 def test_driver_rejects_bad_calls(dev):
     from tensorlib_amd import TensorLibError
     from tensorlib_amd.llama2 import Llama2Config, Llama2Model
