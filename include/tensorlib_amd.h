@@ -115,6 +115,9 @@ int tl_set_hgemm_splits(int splits);
 /* Tuning hook: the MFMA GEMM's workgroups start their walk over K at K tile
  * (tile_column * per_tile + xcd * per_xcd) % tiles and wrap (-1 = automatic, 0 = no rotation). */
 int tl_set_hgemm_k_rotation(int per_tile, int per_xcd);
+/* Tuning hook: the MFMA GEMM numbers its tiles down bands of `band` rows of tiles (0 = automatic; a value of
+ * at least the number of tile rows numbers them down whole columns). */
+int tl_set_hgemm_tile_band(int band);
 /* Tuning hook: prefill attention kernel, 0 = automatic, 1 = one wavefront per 32 query rows,
  * 2 = LDS-tiled workgroups of 128 query rows (head_dim 128, ldv covering the context rounded up to 64). */
 int tl_set_prefill_attention_variant(int variant);

@@ -40,19 +40,34 @@ struct HgemmArgs {
     // Workgroups that run at the same time then touch different column offsets of the 8 KB-strided rows, which
     // spreads their requests over the memory channels (tile-shaped streaming of B from HBM: 4.3 -> 5.9 TB/s).
     int rot_tile, rot_xcd;
+    // Tiles are numbered band by band: a band is band_m rows of tiles over all columns, walked column by column.
+    int band_m;
 };
 
 constexpr int kPad = 8;  // halves of padding per LDS row
 
 // Map the linear workgroup id to a tile so that workgroups resident on one XCD (ids
-// congruent mod 8 are dispatched to the same XCD) work on neighbouring tiles that share a
-// panel of B, and panels of B are walked once.
-__device__ __forceinline__ void tile_of_block(int bid, int nblocks, int tiles_m, int& tm, int& tn) {
-    // XCD x takes a contiguous run of tiles: nblocks / 8 of them, one more on the first nblocks % 8 XCDs
+// congruent mod 8 are dispatched to the same XCD) work on neighbouring tiles: XCD x takes a contiguous run of
+// tile numbers, and tiles are numbered down a band of `band` rows of tiles, column after column, band after
+// band.  The 32 tiles an XCD works on at a time then cover about band x 32/band panels of A and B, which its
+// L2 serves to all of them; with more rows of tiles than `band` a whole column of tiles would share only its
+// panel of B and pull every panel of A through the L2 for a single use.
+__device__ __forceinline__ void tile_of_block(int bid, int nblocks, int tiles_m, int band, int& tm, int& tn) {
+    // nblocks / 8 tiles per XCD, one more on the first nblocks % 8 XCDs
     const int x = bid & 7, base = nblocks >> 3, rem = nblocks & 7;
     const int lid = x * base + (x < rem ? x : rem) + (bid >> 3);
-    tm = lid % tiles_m;
-    tn = lid / tiles_m;
+    if (band >= tiles_m) {
+        tm = lid % tiles_m;
+        tn = lid / tiles_m;
+        return;
+    }
+    const int tiles_n = nblocks / tiles_m;
+    const int per_band = band * tiles_n;
+    const int b = lid / per_band;
+    const int r = lid - b * per_band;
+    const int rows = (tiles_m - b * band) < band ? (tiles_m - b * band) : band;  // the last band may be lower
+    tm = b * band + r % rows;
+    tn = r / rows;
 }
 
 template <int BM, int BN, int BK, int WM, int WN>
@@ -78,7 +93,7 @@ __global__ void __launch_bounds__(WM* WN * 64) hgemm_f16_mfma_kernel(HgemmArgs a
     const int wm = wave / WN, wn = wave % WN;
 
     int tile_m, tile_n;
-    tile_of_block(blockIdx.x, gridDim.x, a.tiles_m, tile_m, tile_n);
+    tile_of_block(blockIdx.x, gridDim.x, a.tiles_m, a.band_m, tile_m, tile_n);
     const int m0 = tile_m * BM, n0 = tile_n * BN;
     const int batch = blockIdx.y;
     const half_t* __restrict__ A = a.A + (size_t)batch * a.sa;
@@ -244,7 +259,8 @@ __global__ void __launch_bounds__(WM* WN * 64) hgemm_f16_dlds_kernel(HgemmArgs a
     // lgkmcnt(0), which also waits for the fragment reads issued just before it.
     float* const partial = a.partial;
     const unsigned rot_tile = (unsigned)a.rot_tile, rot_xcd = (unsigned)a.rot_xcd;
-    asm volatile("" ::"s"(partial), "s"(C), "s"(M), "s"(N), "s"(a.kt_per_split), "s"(rot_tile), "s"(rot_xcd));
+    const int band_m = a.band_m;
+    asm volatile("" ::"s"(partial), "s"(C), "s"(M), "s"(N), "s"(a.kt_per_split), "s"(rot_tile), "s"(rot_xcd), "s"(band_m));
 
     // ---- loader: wavefront-load j of this wavefront covers tile rows (j*NW + wave)*RPW .. +RPW ----
     const int ld_row_in_group = lane / CPR;
@@ -258,7 +274,7 @@ __global__ void __launch_bounds__(WM* WN * 64) hgemm_f16_dlds_kernel(HgemmArgs a
     int rot = 0;  // first K tile of this workgroup's walk (relative to its split)
     auto setup_tile = [&](int b) {
         int tile_m, tile_n;
-        tile_of_block(b, total_tiles, a.tiles_m, tile_m, tile_n);
+        tile_of_block(b, total_tiles, a.tiles_m, band_m, tile_m, tile_n);
         m0 = tile_m * BM;
         n0 = tile_n * BN;
         rot = KT > 0 ? (int)(((unsigned)tile_n * rot_tile + (blockIdx.x & 7u) * rot_xcd) % (unsigned)KT) : 0;
@@ -636,6 +652,7 @@ static bool g_attr_set[kNumVariants] = {false};
 
 static int g_forced_splits = 0;  // 0 = automatic
 static int g_forced_rot_tile = -1, g_forced_rot_xcd = -1;  // -1 = automatic
+static int g_forced_band = 0;                              // 0 = automatic
 
 // Library-owned fp32 workspace for split-K partial sums, grown on demand (stream-ordered reuse).
 static std::mutex g_ws_mu;
@@ -775,6 +792,8 @@ int launch_hgemm(const void* A, const void* B, void* C, size_t M, size_t N, size
     a.partial = nullptr;
     a.rot_tile = 0;
     a.rot_xcd = 0;
+    // band height that balances the panels of A and B an XCD's 32 tiles pull through its L2
+    a.band_m = g_forced_band > 0 ? g_forced_band : (v.bm >= 2 * v.bn ? 4 : 8);
     int splits = 1;
     if (v.stages > 0) {
         // Split K when the tile grid alone cannot occupy the chip (prefill with few tokens: the
@@ -896,6 +915,12 @@ int tl_set_hgemm_k_rotation(int per_tile, int per_xcd) {
     TL_REQUIRE(per_tile >= -1 && per_xcd >= -1, "tl_set_hgemm_k_rotation: negative step");
     tl::g_forced_rot_tile = per_tile;
     tl::g_forced_rot_xcd = per_xcd;
+    return TL_OK;
+}
+
+int tl_set_hgemm_tile_band(int band) {
+    TL_REQUIRE(band >= 0, "tl_set_hgemm_tile_band: negative band");
+    tl::g_forced_band = band;
     return TL_OK;
 }
 

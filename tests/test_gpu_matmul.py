@@ -183,6 +183,34 @@ def test_hgemm_k_rotation_and_splits_visit_every_k_tile_once(dev, oracle):
         dev.lib.tl_set_hgemm_k_rotation(-1, -1)
 
 
+def test_hgemm_tile_bands_cover_every_tile_once(dev):
+    """Tiles are numbered band by band (a band = a few rows of tiles over all columns); whatever the band height,
+    and with a last band that is lower than the others, the numbering must reach every tile.  A carries a row
+    block pattern, B a column block pattern, K = 64: C[i, j] then names its tile, so a tile computed from the
+    wrong panels shows, and a C poisoned beforehand shows a tile that nobody wrote."""
+    names = dev.hgemm_variants()
+    try:
+        for (M, N, name) in [(9 * 256 + 40, 5 * 256 + 8, "p256x256x64w2x4s2"), (19 * 128, 3 * 256, "p128x256x64w2x4s3"),
+                             (11 * 128 + 1, 7 * 128, "t128x128x64w2x2"), (4096 + 256, 2048, "auto")]:
+            A = np.zeros((M, 64), np.float16)
+            B = np.zeros((N, 64), np.float16)
+            A[:, 0] = (np.arange(M) // 128) % 64
+            A[:, 1] = 1
+            B[:, 0] = 1
+            B[:, 1] = (np.arange(N) // 128) % 64
+            want = (A[:, :1].astype(np.float32) + B[:, 1].astype(np.float32)[None, :]).astype(np.float16)
+            Ad, Bd = dev.from_numpy(A), dev.from_numpy(B)
+            dev.set_hgemm_variant(names.index(name))
+            for band in (0, 1, 3, 4, 8, 1000):
+                dev.lib.tl_set_hgemm_tile_band(band)
+                C = torch.full((M, N), -7.0, dtype=torch.float16, device=Ad.device)
+                dev.hgemm(Ad, Bd, C)
+                assert np.array_equal(C.cpu().numpy().view(np.uint16), want.view(np.uint16)), (M, N, name, band)
+    finally:
+        dev.set_hgemm_variant(0)
+        dev.lib.tl_set_hgemm_tile_band(0)
+
+
 def test_hgemm_identity(dev):
     """B = I returns A; A = I returns B^T (catches a transposed operand or tile mapping)."""
     n = 320
