@@ -70,7 +70,7 @@ def cpu_baseline_gemv(budget_s: float = 10.0):
     oracle.matmul2d(mats[0][1], mats[0][0])  # warm-up (thread pool, tables)
     times = []
     t_start = time.perf_counter()
-    while len(times) < 3 or (time.perf_counter() - t_start < budget_s and len(times) < 50):
+    while len(times) < 3 or (time.perf_counter() - t_start < budget_s and len(times) < 5000):
         t0 = time.perf_counter()
         for W, x in mats:
             oracle.matmul2d(x, W)
