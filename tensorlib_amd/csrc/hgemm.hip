@@ -263,14 +263,19 @@ __global__ void __launch_bounds__(WM* WN * 64) hgemm_f16_dlds_kernel(HgemmArgs a
     asm volatile("" ::"s"(partial), "s"(C), "s"(M), "s"(N), "s"(a.kt_per_split), "s"(rot_tile), "s"(rot_xcd), "s"(band_m));
 
     // ---- loader: wavefront-load j of this wavefront covers tile rows (j*NW + wave)*RPW .. +RPW ----
+    // A request's address is a wavefront-uniform base (first row of the tile at the K tile wanted, in scalar
+    // registers) plus a per-lane byte offset that is fixed for the whole C tile, and its LDS target a scalar
+    // too: walking K costs a few scalar instructions per K tile and none per request.
     const int ld_row_in_group = lane / CPR;
     const int ld_slot = lane % CPR;
-    const half_t* a_src[A_LOADS];
-    const half_t* b_src[B_LOADS];
+    unsigned a_voff[A_LOADS], b_voff[B_LOADS];
+    const half_t* a_tile = A;
+    const half_t* b_tile = B;
+    const unsigned lds_wave = (unsigned)(unsigned long)lds + (unsigned)wave * 1024u;
     const int KT_all = K / BK;
     const int kt_begin = (int)blockIdx.z * a.kt_per_split;
     const int KT = (KT_all - kt_begin) < a.kt_per_split ? (KT_all - kt_begin) : a.kt_per_split;
-    // tile `b` of the launch: sets m0, n0 and the per-lane source pointers (at this split's first K tile)
+    // tile `b` of the launch: sets m0, n0, the tile bases (at this split's first K tile) and the lane offsets
     int rot = 0;  // first K tile of this workgroup's walk (relative to its split)
     auto setup_tile = [&](int b) {
         int tile_m, tile_n;
@@ -278,21 +283,21 @@ __global__ void __launch_bounds__(WM* WN * 64) hgemm_f16_dlds_kernel(HgemmArgs a
         m0 = tile_m * BM;
         n0 = tile_n * BN;
         rot = KT > 0 ? (int)(((unsigned)tile_n * rot_tile + (blockIdx.x & 7u) * rot_xcd) % (unsigned)KT) : 0;
+        a_tile = A + (size_t)m0 * K + (size_t)kt_begin * BK;
+        b_tile = B + (size_t)n0 * K + (size_t)kt_begin * BK;
 #pragma unroll
         for (int j = 0; j < A_LOADS; ++j) {
             const int r = (j * NW + wave) * RPW + ld_row_in_group;  // tile row
             const int c = ld_slot ^ ((r / RPL) % CPR);              // chunk of that row this lane fetches
-            int gr = m0 + r;
-            gr = gr < M ? gr : M - 1;
-            a_src[j] = A + (size_t)gr * K + c * 8 + (size_t)kt_begin * BK;
+            const int rr = m0 + r < M ? r : M - 1 - m0;             // rows past the end re-read the last one
+            a_voff[j] = (unsigned)(((size_t)rr * K + c * 8) * sizeof(half_t));
         }
 #pragma unroll
         for (int j = 0; j < B_LOADS; ++j) {
             const int r = (j * NW + wave) * RPW + ld_row_in_group;
             const int c = ld_slot ^ ((r / RPL) % CPR);
-            int gr = n0 + r;
-            gr = gr < N ? gr : N - 1;
-            b_src[j] = B + (size_t)gr * K + c * 8 + (size_t)kt_begin * BK;
+            const int rr = n0 + r < N ? r : N - 1 - n0;
+            b_voff[j] = (unsigned)(((size_t)rr * K + c * 8) * sizeof(half_t));
         }
     };
     int vb = blockIdx.x;
@@ -305,27 +310,18 @@ __global__ void __launch_bounds__(WM* WN * 64) hgemm_f16_dlds_kernel(HgemmArgs a
         k = k >= KT ? k - KT : k;
         return (size_t)k * BK;
     };
-    auto issue_a = [&](int kt) {
-        lds_byte_t* sa = lds + a_off(kt);
-        const size_t koff = k_of(kt);
-#pragma unroll
-        for (int j = 0; j < A_LOADS; ++j)
-            load_16B_per_lane_to_lds(a_src[j] + koff, sa + (j * NW + wave) * 1024);
-    };
-    auto issue_b = [&](int kt) {
-        lds_byte_t* sb = lds + b_off(kt);
-        const size_t koff = k_of(kt);
-#pragma unroll
-        for (int j = 0; j < B_LOADS; ++j)
-            load_16B_per_lane_to_lds(b_src[j] + koff, sb + (j * NW + wave) * 1024);
-    };
-    // wavefront-load l of tile kt: l < A_LOADS from A, the rest from B
-    auto issue_one = [&](int kt, int l) {
-        const size_t koff = k_of(kt);
+    // wavefront-load l of a K tile whose bases and LDS stage the caller has worked out: l < A_LOADS from A
+    auto issue_one_at = [&](const half_t* abase, const half_t* bbase, unsigned stage, int l) {
         if (l < A_LOADS)
-            load_16B_per_lane_to_lds(a_src[l] + koff, lds + a_off(kt) + (l * NW + wave) * 1024);
+            load_16B_per_lane_to_lds(abase, a_voff[l], stage + (unsigned)(l * NW * 1024));
         else
-            load_16B_per_lane_to_lds(b_src[l - A_LOADS] + koff, lds + b_off(kt) + ((l - A_LOADS) * NW + wave) * 1024);
+            load_16B_per_lane_to_lds(bbase, b_voff[l - A_LOADS], stage + (unsigned)(A_BYTES + (l - A_LOADS) * NW * 1024));
+    };
+    auto issue_tile = [&](int kt) {
+        const size_t koff = k_of(kt);
+        const unsigned stage = lds_wave + (unsigned)a_off(kt);
+#pragma unroll
+        for (int l = 0; l < LPW; ++l) issue_one_at(a_tile + koff, b_tile + koff, stage, l);
     };
 
     // ---- fragment reader: row (lane % 32) of a 32-row MFMA tile, chunk 2*ks + lane/32 ----
@@ -340,7 +336,7 @@ __global__ void __launch_bounds__(WM* WN * 64) hgemm_f16_dlds_kernel(HgemmArgs a
     float16_t acc[MT][NT];
 #pragma unroll
     for (int s = 0; s < STAGES - 1; ++s)
-        if (s < KT) { issue_a(s); issue_b(s); }
+        if (s < KT) issue_tile(s);
 
     // Wait until tile kt has landed in LDS for every wavefront.  Tiles requested after kt
     // (at most STAGES-2 of them) may stay in flight.
@@ -353,17 +349,21 @@ __global__ void __launch_bounds__(WM* WN * 64) hgemm_f16_dlds_kernel(HgemmArgs a
     };
     // After the barrier of tile kt every wavefront is done with tile kt-1: refill what it occupied.
     auto issue_after_sync = [&](int kt) {
-        if (kt + STAGES - 1 < KT) { issue_a(kt + STAGES - 1); issue_b(kt + STAGES - 1); }
+        if (kt + STAGES - 1 < KT) issue_tile(kt + STAGES - 1);
     };
+    // Fragment reads go out in the order the MFMAs of a step (A index outer, B index inner) first need them:
+    // A0, B0 .. B(NT-1), A1 .. A(MT-1).  LDS returns data in order, so the wait in front of an MFMA then counts
+    // only the reads that MFMA needs, and each read has had most of a step to land.
     auto load_frags = [&](half8_t (&af)[MT], half8_t (&bf)[NT], int kt, int ks) {
         const unsigned char* sa = smem_raw + a_off(kt) + a_base;
         const unsigned char* sb = smem_raw + b_off(kt) + b_base;
-#pragma unroll
-        for (int i = 0; i < MT; ++i)
-            af[i] = *reinterpret_cast<const half8_t*>(sa + i * 32 * RB + fr_off[ks]);
+        af[0] = *reinterpret_cast<const half8_t*>(sa + fr_off[ks]);
 #pragma unroll
         for (int j = 0; j < NT; ++j)
             bf[j] = *reinterpret_cast<const half8_t*>(sb + j * 32 * RB + fr_off[ks]);
+#pragma unroll
+        for (int i = 1; i < MT; ++i)
+            af[i] = *reinterpret_cast<const half8_t*>(sa + i * 32 * RB + fr_off[ks]);
     };
     auto mfmas = [&](const half8_t (&af)[MT], const half8_t (&bf)[NT]) {
 #pragma unroll
@@ -385,62 +385,93 @@ __global__ void __launch_bounds__(WM* WN * 64) hgemm_f16_dlds_kernel(HgemmArgs a
             for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
 
     if constexpr (MODE == 1) {
-        // Fragments are double buffered in registers: the ds_reads of K step s+1 (or of the
-        // next tile's first step, after the tile barrier) are issued before the MFMAs of step s.
+        // Fragments are double buffered in registers: the ds_reads of K step s+1 (or of the next tile's first
+        // step, after the tile barrier) go out one by one behind the first MFMAs of step s, in the order
+        // load_frags uses.
+        //
+        // Where the requests that refill the ring go.  With three or more stages they are spread over a whole K
+        // tile of MFMAs: segment 0 of a tile's LPW requests goes out in the last step of the tile that frees
+        // its stage (after the barrier), segments 1 .. KS-1 in steps 0 .. KS-2 of the next tile; all of them
+        // are older than that next tile's barrier, so the vmcnt counts do not change.  With two stages a tile
+        // has one K tile of time to land, and spreading its requests made every barrier wait 400-570 cycles
+        // for data (measured), so there all LPW requests go out behind the MFMAs of the last step.
         static_assert(KS % 2 == 0, "fragment ping-pong needs an even number of K steps");
+        constexpr int NM = MT * NT;
         half8_t af[2][MT], bf[2][NT];
+        // requests [seg * LPW / KS, (seg + 1) * LPW / KS) of K tile kt, request i of them behind MFMA m
+        constexpr bool SPREAD = STAGES >= 3;
+        auto issue_segment = [&](int seg, int m, const half_t* abase, const half_t* bbase, unsigned stage) {
+            const int l0 = SPREAD ? seg * LPW / KS : (seg == 0 ? 0 : LPW);
+            const int l1 = SPREAD ? (seg + 1) * LPW / KS : LPW;
+            const int n = l1 - l0;
+#pragma unroll
+            for (int i = 0; i < n; ++i) {
+                const int at = n <= NM ? i * (NM / n) + (NM / n) / 2 : i % NM;
+                if (at == m) issue_one_at(abase, bbase, stage, l0 + i);
+            }
+        };
         sync_for(0);
-        issue_after_sync(0);
+        if (STAGES - 1 < KT) {  // segment 0 of the tile that follows the prologue's; the rest inside tile(0)
+            const size_t koff = k_of(STAGES - 1);
+#pragma unroll
+            for (int m = 0; m < NM; ++m) issue_segment(0, m, a_tile + koff, b_tile + koff, lds_wave + (unsigned)a_off(STAGES - 1));
+        }
         load_frags(af[0], bf[0], 0, 0);
-        // The last tile is peeled off so that inside the loop the fragments of the next tile are always
-        // requested: the compiler then knows how many reads are younger than the ones an MFMA needs.
-        auto tile = [&](int kt, auto has_next) {
+        // has_next: another K tile follows (its first fragments are requested in the last step);
+        // fill: K tile kt + STAGES - 1 exists (its segments 1.. go out in steps 0 .. KS-2);
+        // more: K tile kt + STAGES exists (its segment 0 goes out in the last step).
+        // All compile-time, and the last K tile is peeled off, so every step is straight-line code and the
+        // compiler knows how many reads are younger than the ones an MFMA needs.
+        auto tile = [&](int kt, auto has_next, auto fill, auto more) {
+            const size_t koff_fill = decltype(fill)::value ? k_of(kt + STAGES - 1) : 0;
+            const half_t* abase_fill = a_tile + koff_fill;
+            const half_t* bbase_fill = b_tile + koff_fill;
+            const unsigned stage_fill = lds_wave + (unsigned)a_off(kt + STAGES - 1);
 #pragma unroll
             for (int ks = 0; ks < KS; ++ks) {
                 const int cur = ks & 1, nxt = cur ^ 1;
-                if (ks + 1 < KS) {
-                    load_frags(af[nxt], bf[nxt], kt, ks + 1);
-                } else if constexpr (decltype(has_next)::value) {
-                    // Last step of the tile: after the barrier the matrix core restarts at once, and the
-                    // requests for the tile after next and the first fragment reads of the next tile go out
-                    // one by one behind the MFMAs instead of in a block in front of them.
-                    sync_for(kt + 1);  // every wavefront holds its last fragments of tile kt in registers
-                    const bool more = kt + STAGES < KT;
-                    constexpr int NM = MT * NT;
-                    const unsigned char* sa = smem_raw + a_off(kt + 1) + a_base;
-                    const unsigned char* sb = smem_raw + b_off(kt + 1) + b_base;
-#pragma unroll
-                    for (int m = 0; m < NM; ++m) {
-                        const int i = m / NT, j = m % NT;
-                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(bf[cur][j], af[cur][i], acc[i][j], 0, 0, 0);
-#pragma unroll
-                        for (int r = m; r < MT + NT; r += NM) {
-                            if (r < MT) af[nxt][r] = *reinterpret_cast<const half8_t*>(sa + r * 32 * RB + fr_off[0]);
-                            else bf[nxt][r - MT] = *reinterpret_cast<const half8_t*>(sb + (r - MT) * 32 * RB + fr_off[0]);
-                        }
-                        if (more) {
-#pragma unroll
-                            for (int l = m; l < LPW; l += NM) issue_one(kt + STAGES, l);
-                        }
-                        __builtin_amdgcn_sched_barrier(0);
-                    }
+                const bool last = ks + 1 == KS;
+                if (last && !decltype(has_next)::value) {
+                    mfmas(af[cur], bf[cur]);
                     continue;
                 }
-                mfmas(af[cur], bf[cur]);
-                // Issue order inside the step: one fragment read of the next step behind each of the first
-                // MFMAs (an MFMA occupies the matrix core for 32 cycles but its issue slot for 4, so the reads
-                // go out under it and land under the rest of the step), nothing crosses into the next step.
+                // where the fragments of the next step live: this tile's stage, or the next tile's after its barrier
+                if (last) sync_for(kt + 1);  // every wavefront holds its last fragments of tile kt in registers
+                const int rk = last ? kt + 1 : kt, rs = last ? 0 : ks + 1;
+                const unsigned char* sa = smem_raw + a_off(rk) + a_base;
+                const unsigned char* sb = smem_raw + b_off(rk) + b_base;
+                const size_t koff = (last && decltype(more)::value) ? k_of(kt + STAGES) : 0;
+                const half_t* abase = last ? a_tile + koff : abase_fill;
+                const half_t* bbase = last ? b_tile + koff : bbase_fill;
+                const unsigned stage = last ? lds_wave + (unsigned)a_off(kt + STAGES) : stage_fill;
 #pragma unroll
-                for (int r = 0; r < MT + NT; ++r) {
-                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // 1 MFMA
-                    __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // 1 LDS read
+                for (int m = 0; m < NM; ++m) {
+                    const int i = m / NT, j = m % NT;
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(bf[cur][j], af[cur][i], acc[i][j], 0, 0, 0);
+#pragma unroll
+                    for (int r = m; r < MT + NT; r += NM) {  // same order as load_frags
+                        if (r == 0) af[nxt][0] = *reinterpret_cast<const half8_t*>(sa + fr_off[rs]);
+                        else if (r <= NT) bf[nxt][r - 1] = *reinterpret_cast<const half8_t*>(sb + (r - 1) * 32 * RB + fr_off[rs]);
+                        else af[nxt][r - NT] = *reinterpret_cast<const half8_t*>(sa + (r - NT) * 32 * RB + fr_off[rs]);
+                    }
+                    if (last) {
+                        if constexpr (decltype(more)::value) issue_segment(0, m, abase, bbase, stage);
+                    } else {
+                        if constexpr (decltype(fill)::value) issue_segment(ks + 1, m, abase, bbase, stage);
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
                 }
-                __builtin_amdgcn_sched_group_barrier(0x008, MT * NT - (MT + NT), 0);
-                __builtin_amdgcn_sched_barrier(0);
             }
         };
-        for (int kt = 0; kt + 1 < KT; ++kt) tile(kt, std::true_type{});
-        if (KT > 0) tile(KT - 1, std::false_type{});
+        {
+            using T = std::true_type;
+            using F = std::false_type;
+            int kt = 0;
+            for (; kt + STAGES < KT; ++kt) tile(kt, T{}, T{}, T{});
+            for (; kt + STAGES - 1 < KT && kt + 1 < KT; ++kt) tile(kt, T{}, T{}, F{});
+            for (; kt + 1 < KT; ++kt) tile(kt, T{}, F{}, F{});
+            if (KT > 0) tile(KT - 1, F{}, F{}, F{});
+        }
     } else {
         for (int kt = 0; kt < KT; ++kt) {
             sync_for(kt);
@@ -475,7 +506,7 @@ __global__ void __launch_bounds__(WM* WN * 64) hgemm_f16_dlds_kernel(HgemmArgs a
             setup_tile(next_vb);
 #pragma unroll
             for (int st = 0; st < STAGES - 1; ++st)
-                if (st < KT) { issue_a(st); issue_b(st); }
+                if (st < KT) issue_tile(st);
             stage_area = (STAGES - 1) * STAGE_BYTES;
         }
     }
@@ -767,6 +798,8 @@ int launch_hgemm(const void* A, const void* B, void* C, size_t M, size_t N, size
     }
     int vi = g_forced_variant ? g_forced_variant : pick_variant(M, N, K, device_info().cu_count);
     if (g_variants[vi].stages > 0 && K % g_variants[vi].bk != 0) vi = 1;  // direct-to-LDS path cannot zero-fill a K tail
+    // its per-lane byte offsets inside a tile ((rows - 1) * K + 64 halves) are 32-bit
+    if (g_variants[vi].stages > 0 && K > ((size_t)1 << 22)) vi = 1;
     const HgemmVariant& v = g_variants[vi];
     const size_t lds = lds_bytes(v);
     if (lds > 64 * 1024 && !g_attr_set[vi]) {

@@ -71,6 +71,15 @@ __device__ __forceinline__ void load_16B_per_lane_to_lds(const half_t* src,
     asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(src), "s"(lds_addr) : "memory");
 }
 
+// The same instruction with the address split into a wavefront-uniform base (a scalar register pair) and a
+// 32-bit byte offset per lane: a tile's per-lane offsets stay put while only the base moves along K, so a
+// request costs no vector arithmetic.
+__device__ __forceinline__ void load_16B_per_lane_to_lds(const void* uniform_base, unsigned lane_offset,
+                                                         unsigned lds_addr) {
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %0"
+                 ::"s"(uniform_base), "v"(lane_offset), "s"(lds_addr) : "memory");
+}
+
 template <int N_>
 __device__ __forceinline__ void wait_vmcnt_and_barrier() {
     // waits until at most N_ of this wavefront's global->LDS loads are outstanding and all of its
