@@ -148,6 +148,16 @@ def test_hgemm_unaligned_k(dev, oracle, M, N, K):
     _hgemm_case(dev, oracle, M, N, K, seed=1100 + K, b_std=0.1)
 
 
+def test_hgemm_rows_longer_than_the_ring_kernels_address(dev, oracle):
+    """The direct-to-LDS kernels address a tile's rows with 32-bit byte offsets, good for K up to 2^22; a longer
+    K (still a multiple of 64) must be routed to the register-staged kernel and come out right."""
+    M, N, K = 4, 16, (1 << 22) + 64
+    A = synth.normal_f16(1190, (M, K), 0.05)
+    B = synth.normal_f16(1191, (N, K), 0.05)
+    C = dev.hgemm(dev.from_numpy(A), dev.from_numpy(B)).cpu().numpy()
+    assert_close_f16(C, oracle.matmul2d(A, B), RTOL, ATOL, "hgemm K = 2^22 + 64")
+
+
 def test_hgemm_integer_inputs_bit_exact(dev, oracle):
     M, N, K = 256, 384, 512
     A = synth.small_ints_f16(1200, (M, K), -2, 2)
