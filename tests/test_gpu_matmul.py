@@ -278,6 +278,25 @@ def test_matmul_error_behaviour(dev):
         dev.matmul(a, dev.empty(5, 3), out=dev.empty(4, 4))
 
 
+def test_matmul2d_degenerate_sizes(dev):
+    """M == 0 or N == 0: nothing to write; K == 0: the empty sum, i.e. zeros (CPU<half>::matmul2d's loop over k does
+    not run, tensorLib/src/device/cpu/CPU.cpp:76-89) -- for the GEMV (M == 1) and the GEMM path alike."""
+    import ctypes
+    A = torch.ones(8, 16, dtype=torch.float16, device="cuda")
+    B = torch.ones(24, 16, dtype=torch.float16, device="cuda")
+    vp = lambda t: ctypes.c_void_p(t.data_ptr())
+    for (M, N) in [(0, 24), (8, 0), (0, 0), (1, 0)]:
+        C = torch.full((8, 24), -7.0, dtype=torch.float16, device="cuda")
+        assert dev.lib.tl_matmul2d_f16(vp(A), vp(B), vp(C), M, N, 16) == 0
+        torch.cuda.synchronize()
+        assert bool((C == -7.0).all()), (M, N)
+    for M in (1, 8):
+        C = torch.full((M, 24), -7.0, dtype=torch.float16, device="cuda")
+        assert dev.lib.tl_matmul2d_f16(vp(A), vp(B), vp(C), M, 24, 0) == 0
+        torch.cuda.synchronize()
+        assert bool((C == 0).all()), M
+
+
 def test_matmul2d_f32(dev, oracle):
     rng = np.random.default_rng(11)
     for (M, N, K) in [(1, 1, 1), (17, 33, 65), (128, 100, 300)]:
