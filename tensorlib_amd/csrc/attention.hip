@@ -41,18 +41,16 @@ constexpr int kAttnChunk = 64;  // cached positions per workgroup
 
 // partial layout per (head, chunk): [0] = max, [1] = sum, [2 .. 2+head_dim) = sum_t p_t * V[t]
 // Rotate the 4 (even, odd) pairs of one 16-byte chunk of a head vector; `d0` is the index of the
-// chunk's first element inside the head.  Same arithmetic as rope_kernel: fp32 angle, cos/sin
-// rounded to half, fp32 products, one rounding per output.
+// chunk's first element inside the head.  Same arithmetic as rope_kernel (rope_cos_sin, rope_rotate).
 __device__ __forceinline__ half8_t rope_chunk(half8_t v, int pos, int d0, int head_dim) {
     half8_t r;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-        const float theta = (float)pos * 1.0f / powf(10000.0f, (float)(d0 + 2 * i) / (float)head_dim);
-        const float c = (float)(half_t)cosf(theta);
-        const float s = (float)(half_t)sinf(theta);
-        const float v0 = (float)v[2 * i], v1 = (float)v[2 * i + 1];
-        r[2 * i] = (half_t)(v0 * c - v1 * s);
-        r[2 * i + 1] = (half_t)(v0 * s + v1 * c);
+        float c, s;
+        rope_cos_sin(pos, d0 + 2 * i, head_dim, c, s);
+        const half2_t o = rope_rotate((float)v[2 * i], (float)v[2 * i + 1], c, s);
+        r[2 * i] = o[0];
+        r[2 * i + 1] = o[1];
     }
     return r;
 }
@@ -62,30 +60,32 @@ __device__ __forceinline__ half8_t rope_chunk_cs(half8_t v, half8_t cs) {
     half8_t r;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-        const float c = (float)cs[2 * i], s = (float)cs[2 * i + 1];
-        const float v0 = (float)v[2 * i], v1 = (float)v[2 * i + 1];
-        r[2 * i] = (half_t)(v0 * c - v1 * s);
-        r[2 * i + 1] = (half_t)(v0 * s + v1 * c);
+        const half2_t o = rope_rotate((float)v[2 * i], (float)v[2 * i + 1], (float)cs[2 * i], (float)cs[2 * i + 1]);
+        r[2 * i] = o[0];
+        r[2 * i + 1] = o[1];
     }
     return r;
 }
 
-// table[pos][pair] = (half(cos(theta)), half(sin(theta))), theta = pos / 10000^(2*pair/head_dim) in fp32:
-// the values every RoPE kernel of this library computes on the fly.
+// table[pos][pair] = (half(cos(theta)), half(sin(theta))), theta = pos / 10000^(2*pair/head_dim) in fp32
+// (rope_cos_sin): the values every RoPE kernel of this library computes on the fly.
 __global__ void __launch_bounds__(256) rope_table_kernel(half_t* table, int max_seq, int head_dim) {
     const int half_d = head_dim / 2;
     const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= (size_t)max_seq * half_d) return;
     const int pos = (int)(i / half_d), pair = (int)(i % half_d);
-    const float theta = (float)pos * 1.0f / powf(10000.0f, (float)(2 * pair) / (float)head_dim);
-    half2_t cs = {(half_t)cosf(theta), (half_t)sinf(theta)};
+    float c, s;
+    rope_cos_sin(pos, 2 * pair, head_dim, c, s);
+    half2_t cs = {(half_t)c, (half_t)s};
     *reinterpret_cast<half2_t*>(table + 2 * i) = cs;
 }
 
 // FUSE_ROPE: `q` points at the raw q|k|v projection of the new token (position T-1).  q is rotated
 // on load; the workgroup that owns the last chunk rotates the new k row, uses it, and writes it and
 // the new v row into the caches (each head's workgroup writes only its own head slice).
-template <int LPR, bool FUSE_ROPE>
+// ROPE: 0 = q is already rotated and the caches hold position T-1; 1 = rotate with the table's (cos, sin);
+// 2 = rotate with cos/sin evaluated in the kernel (no table given).
+template <int LPR, int ROPE>
 __global__ void __launch_bounds__(kAttnThreads)
 decode_attn_partial_kernel(half_t* out, float* partial, const half_t* q, half_t* cache_k,
                            half_t* cache_v, const half_t* rope_table, int T, int n_heads, float inv_scale,
@@ -107,13 +107,12 @@ decode_attn_partial_kernel(half_t* out, float* partial, const half_t* q, half_t*
 
     half8_t qv = *reinterpret_cast<const half8_t*>(q + (size_t)h * D + sub * 8);
     half8_t cs = {0, 0, 0, 0, 0, 0, 0, 0};  // (cos, sin) of the 4 pairs of this thread's chunk at position T-1
-    if constexpr (FUSE_ROPE) {
-        if (rope_table) {
-            cs = *reinterpret_cast<const half8_t*>(rope_table + ((size_t)(T - 1) * (D / 2) + sub * 4) * 2);
-            qv = rope_chunk_cs(qv, cs);
-        } else {
-            qv = rope_chunk(qv, T - 1, sub * 8, D);
-        }
+    constexpr bool FUSE_ROPE = ROPE != 0;
+    if constexpr (ROPE == 1) {
+        cs = *reinterpret_cast<const half8_t*>(rope_table + ((size_t)(T - 1) * (D / 2) + sub * 4) * 2);
+        qv = rope_chunk_cs(qv, cs);
+    } else if constexpr (ROPE == 2) {
+        qv = rope_chunk(qv, T - 1, sub * 8, D);
     }
 
     // All K and V rows this thread will touch are requested up front (NIT rows each), so the whole
@@ -145,7 +144,8 @@ decode_attn_partial_kernel(half_t* out, float* partial, const half_t* q, half_t*
         const int t = t0 + grp + it * GROUPS;
         if (t < t1) {
             if (FUSE_ROPE && t == T - 1) {
-                kreg[it] = rope_table ? rope_chunk_cs(kreg[it], cs) : rope_chunk(kreg[it], T - 1, sub * 8, D);
+                if constexpr (ROPE == 1) kreg[it] = rope_chunk_cs(kreg[it], cs);
+                else kreg[it] = rope_chunk(kreg[it], T - 1, sub * 8, D);
                 *reinterpret_cast<half8_t*>(cache_k + (size_t)t * row_stride + head_off) = kreg[it];
                 *reinterpret_cast<half8_t*>(cache_v + (size_t)t * row_stride + head_off) = vreg[it];
             }
@@ -295,8 +295,8 @@ prefill_rope_qkv_kernel(half_t* q_out, const half_t* q, const half_t* k, const h
     const half2_t qv = *reinterpret_cast<const half2_t*>(q + in_off);
     const half2_t kv = *reinterpret_cast<const half2_t*>(k + in_off);
     const half2_t vv = *reinterpret_cast<const half2_t*>(v + in_off);
-    half2_t qr = {(half_t)((float)qv[0] * c - (float)qv[1] * sn), (half_t)((float)qv[0] * sn + (float)qv[1] * c)};
-    half2_t kr = {(half_t)((float)kv[0] * c - (float)kv[1] * sn), (half_t)((float)kv[0] * sn + (float)kv[1] * c)};
+    const half2_t qr = rope_rotate((float)qv[0], (float)qv[1], c, sn);
+    const half2_t kr = rope_rotate((float)kv[0], (float)kv[1], c, sn);
     *reinterpret_cast<half2_t*>(q_out + ((size_t)h * n_tokens + s) * head_dim + 2 * pair) = qr;
     const size_t c_off = ((size_t)(start_pos + s) * n_heads + h) * head_dim + 2 * pair;
     *reinterpret_cast<half2_t*>(cache_k + c_off) = kr;
@@ -718,12 +718,9 @@ rope_qk_store_kv_kernel(half_t* qkv, half_t* cache_k, half_t* cache_v, int pos, 
     half2_t v = *reinterpret_cast<const half2_t*>(qkv + which * dim + e);
     if (which < 2) {
         const int d = e % head_dim;
-        const float theta = (float)pos * 1.0f / powf(10000.0f, (float)d / (float)head_dim);
-        const float c = (float)(half_t)cosf(theta);
-        const float s = (float)(half_t)sinf(theta);
-        const float v0 = (float)v[0], v1 = (float)v[1];
-        v[0] = (half_t)(v0 * c - v1 * s);
-        v[1] = (half_t)(v0 * s + v1 * c);
+        float c, s;
+        rope_cos_sin(pos, d, head_dim, c, s);
+        v = rope_rotate((float)v[0], (float)v[1], c, s);
     }
     if (which == 0)
         *reinterpret_cast<half2_t*>(qkv + e) = v;
@@ -893,14 +890,18 @@ static int launch_decode_attention(void* out, const void* q, void* cache_k, void
                            (const tl::half_t*)q, (tl::half_t*)cache_k, (tl::half_t*)cache_v,
                            (const tl::half_t*)rope_table, T, n_heads, inv_scale, n_chunks);
     };
-    if (fuse_rope) {
-        if (head_dim == 64) launch(tl::decode_attn_partial_kernel<8, true>);
-        else if (head_dim == 128) launch(tl::decode_attn_partial_kernel<16, true>);
-        else launch(tl::decode_attn_partial_kernel<32, true>);
+    if (fuse_rope && rope_table) {
+        if (head_dim == 64) launch(tl::decode_attn_partial_kernel<8, 1>);
+        else if (head_dim == 128) launch(tl::decode_attn_partial_kernel<16, 1>);
+        else launch(tl::decode_attn_partial_kernel<32, 1>);
+    } else if (fuse_rope) {
+        if (head_dim == 64) launch(tl::decode_attn_partial_kernel<8, 2>);
+        else if (head_dim == 128) launch(tl::decode_attn_partial_kernel<16, 2>);
+        else launch(tl::decode_attn_partial_kernel<32, 2>);
     } else {
-        if (head_dim == 64) launch(tl::decode_attn_partial_kernel<8, false>);
-        else if (head_dim == 128) launch(tl::decode_attn_partial_kernel<16, false>);
-        else launch(tl::decode_attn_partial_kernel<32, false>);
+        if (head_dim == 64) launch(tl::decode_attn_partial_kernel<8, 0>);
+        else if (head_dim == 128) launch(tl::decode_attn_partial_kernel<16, 0>);
+        else launch(tl::decode_attn_partial_kernel<32, 0>);
     }
     TL_CHECK_LAUNCH("decode_attn_partial_kernel");
     if (n_chunks > 1) {

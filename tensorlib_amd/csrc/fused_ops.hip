@@ -108,14 +108,10 @@ rope_kernel(const half_t* in, half_t* out, int start_pos, int T, int n_heads, in
     const size_t bth = p / half_d;           // (b*T + t)*H + h
     const int t = (int)((bth / n_heads) % T);
     const int d = dp * 2;
-    const float theta = (float)(start_pos + t) * 1.0f / powf(10000.0f, (float)d / (float)head_dim);
-    const float c = (float)(half_t)cosf(theta);
-    const float s = (float)(half_t)sinf(theta);
+    float c, s;
+    rope_cos_sin(start_pos + t, d, head_dim, c, s);
     const half2_t v = *reinterpret_cast<const half2_t*>(in + 2 * p);
-    const float v0 = (float)v[0], v1 = (float)v[1];
-    half2_t r;
-    r[0] = (half_t)(v0 * c - v1 * s);
-    r[1] = (half_t)(v0 * s + v1 * c);
+    const half2_t r = rope_rotate((float)v[0], (float)v[1], c, s);
     *reinterpret_cast<half2_t*>(out + 2 * p) = r;
 }
 

@@ -80,6 +80,23 @@ __device__ __forceinline__ void load_16B_per_lane_to_lds(const void* uniform_bas
                  ::"s"(uniform_base), "v"(lane_offset), "s"(lds_addr) : "memory");
 }
 
+// Rotary embedding, with every rounding of the reference's CPU loop (tensorLib/src/device/cpu/CPU.cpp:444-453):
+// the angle is an fp32 quotient, cos and sin are rounded to half, each of the four products is rounded to half
+// and so are their difference and sum.  cos, sin and the power are evaluated in double and rounded to fp32 once,
+// i.e. they are the correctly rounded fp32 values a host libm returns for the same fp32 argument.
+__device__ __forceinline__ void rope_cos_sin(int pos, int d, int head_dim, float& c, float& s) {
+    const float base = (float)pow(10000.0, (double)((float)d / (float)head_dim));
+    const float theta = (float)pos * 1.0f / base;
+    c = (float)(half_t)(float)cos((double)theta);
+    s = (float)(half_t)(float)sin((double)theta);
+}
+__device__ __forceinline__ half2_t rope_rotate(float v0, float v1, float c, float s) {
+    const float p0 = (float)(half_t)(v0 * c), p1 = (float)(half_t)(v1 * s);
+    const float p2 = (float)(half_t)(v0 * s), p3 = (float)(half_t)(v1 * c);
+    half2_t r = {(half_t)(p0 - p1), (half_t)(p2 + p3)};
+    return r;
+}
+
 template <int N_>
 __device__ __forceinline__ void wait_vmcnt_and_barrier() {
     // waits until at most N_ of this wavefront's global->LDS loads are outstanding and all of its

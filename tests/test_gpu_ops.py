@@ -35,7 +35,8 @@ def test_rms_norm_in_place(dev, oracle):
 def test_rope(dev, oracle, B, T, H, D, start):
     x = synth.normal_f16(20, (B, T, H, D), 1.0)
     got = dev.apply_rotary_emb(dev.from_numpy(x), start).cpu().numpy()
-    assert_close_f16(got, oracle.rope(x, start), RTOL, 2e-3, "rope")
+    # every rounding of CPU.cpp:444-453 is reproduced, so the gate is bit equality
+    assert np.array_equal(got.view(np.uint16), oracle.rope(x, start).view(np.uint16)), "rope differs from the CPU loop"
     xd = dev.from_numpy(x)
     dev.apply_rotary_emb(xd, start, out=xd)  # in place, as Attention::forward does
     assert np.array_equal(xd.cpu().numpy().view(np.uint16), got.view(np.uint16))
@@ -218,10 +219,10 @@ def test_rope_qk_store_kv(dev, oracle, H, D, pos):
     q_want = oracle.rope(qkv[0].reshape(1, 1, H, D), pos).reshape(H, D)
     k_want = oracle.rope(qkv[1].reshape(1, 1, H, D), pos).reshape(H, D)
     got = qd.cpu().numpy()
-    assert_close_f16(got[0], q_want, RTOL, 2e-3, "q rope")
+    assert np.array_equal(got[0].view(np.uint16), q_want.view(np.uint16)), "q rope"
     assert np.array_equal(got[1:].view(np.uint16), qkv[1:].view(np.uint16))      # k, v inputs untouched
     ck, cv = kd.cpu().numpy(), vd.cpu().numpy()
-    assert_close_f16(ck[pos], k_want, RTOL, 2e-3, "k rope into cache")
+    assert np.array_equal(ck[pos].view(np.uint16), k_want.view(np.uint16)), "k rope into cache"
     assert np.array_equal(cv[pos].view(np.uint16), qkv[2].view(np.uint16))
     keep = np.arange(S) != pos
     assert np.array_equal(ck[keep].view(np.uint16), ck0[keep].view(np.uint16))
@@ -348,6 +349,18 @@ def test_rope_table_values(dev):
     assert np.all(tab[0, :, 0] == 1.0) and np.all(tab[0, :, 1] == 0.0)
 
 
+@pytest.mark.parametrize("D", [128, 64])
+def test_rope_table_bits_equal_the_cpu_loop_at_every_position(dev, oracle, D):
+    """Rotating the pair (1, 0) with the CPU loop returns (half(cos), half(sin)) of its fp32 angle: the table
+    must hold exactly those bits for all 2048 positions of the largest context."""
+    S = 2048
+    ones = np.zeros((1, S, 1, D), np.float16)
+    ones[..., 0::2] = 1.0
+    want = oracle.rope(ones, 0).reshape(S, D // 2, 2)
+    tab = dev.rope_table(S, D).cpu().numpy().reshape(S, D // 2, 2)
+    assert np.array_equal(tab.view(np.uint16), want.view(np.uint16))
+
+
 def test_decode_attention_repeated_calls_reuse_counters(dev, oracle):
     """Many calls in a row with different numbers of chunks share one partials workspace: all of
     them have to agree with the CPU chain."""
@@ -383,9 +396,9 @@ def test_prefill_rope_qkv(dev, oracle, S, H, D, start, fused_rows):
     else:
         qd, kk, vv = (dev.from_numpy(np.ascontiguousarray(a)) for a in (q, k, v))
     got_q = dev.prefill_rope_qkv(qd, kk, vv, kd, vd, table, start, H).cpu().numpy()   # [H, S, D]
-    assert_close_f16(got_q, want_q.transpose(1, 0, 2), RTOL, 2e-3, "prefill rope q")
+    assert np.array_equal(got_q.view(np.uint16), np.ascontiguousarray(want_q.transpose(1, 0, 2)).view(np.uint16)), "prefill rope q"
     gk, gv = kd.cpu().numpy(), vd.cpu().numpy()
-    assert_close_f16(gk[start:start + S], want_k, RTOL, 2e-3, "prefill rope k -> cache")
+    assert np.array_equal(gk[start:start + S].view(np.uint16), want_k.view(np.uint16)), "prefill rope k -> cache"
     assert np.array_equal(gv[start:start + S].view(np.uint16), np.ascontiguousarray(v).reshape(S, H, D).view(np.uint16))
     keep = np.r_[0:start, start + S:T]                                                   # other cache rows untouched
     assert np.array_equal(gk[keep].view(np.uint16), ck0[keep].view(np.uint16))
