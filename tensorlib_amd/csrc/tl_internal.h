@@ -87,10 +87,15 @@ __device__ __forceinline__ void load_16B_per_lane_to_lds(const void* uniform_bas
 __device__ __forceinline__ void rope_cos_sin(int pos, int d, int head_dim, float& c, float& s) {
     const float base = (float)pow(10000.0, (double)((float)d / (float)head_dim));
     const float theta = (float)pos * 1.0f / base;
-    c = (float)(half_t)(float)cos((double)theta);
-    s = (float)(half_t)(float)sin((double)theta);
+    float cf = (float)cos((double)theta), sf = (float)sin((double)theta);
+    // the reference rounds double -> fp32 -> half; without this the compiler merges the two conversions into one
+    // double -> half rounding, which differs when the fp32 value lands on a half-way point
+    asm volatile("" : "+v"(cf), "+v"(sf));
+    c = (float)(half_t)cf;
+    s = (float)(half_t)sf;
 }
 __device__ __forceinline__ half2_t rope_rotate(float v0, float v1, float c, float s) {
+#pragma clang fp contract(off)  // a fused multiply-add would skip the rounding of the second product
     const float p0 = (float)(half_t)(v0 * c), p1 = (float)(half_t)(v1 * s);
     const float p2 = (float)(half_t)(v0 * s), p3 = (float)(half_t)(v1 * c);
     half2_t r = {(half_t)(p0 - p1), (half_t)(p2 + p3)};
