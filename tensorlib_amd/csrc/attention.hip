@@ -11,6 +11,7 @@
 // tl_causal_mask_f16: the additive mask of Transformer::get_mask
 // (model/llama2_7b/src/Transformer.cpp:231-261) written by one kernel instead of one
 // host-to-device copy per element.
+#include <atomic>
 #include <mutex>
 
 #include "tl_internal.h"
@@ -18,7 +19,7 @@
 namespace tl {
 
 // 0: automatic, 1: one wavefront per 32 query rows, 2: LDS-tiled workgroups of 128 query rows (tuning hook)
-static int g_prefill_attention_variant = 0;
+static std::atomic<int> g_prefill_attention_variant{0};
 
 template <int CTRL>
 __device__ __forceinline__ float dppf(float v) {
@@ -833,31 +834,7 @@ add_rms_norm_vec_kernel(half_t* sum_out, half_t* norm_out, const half_t* a, cons
 }
 
 // Library-owned fp32 workspace for the chunk partials, grown on demand.
-static std::mutex g_ws_mu;
-static float* g_ws = nullptr;
-static size_t g_ws_floats = 0;
-
-static int workspace(size_t floats, float** out) {
-    std::lock_guard<std::mutex> lk(g_ws_mu);
-    if (floats > g_ws_floats) {
-        if (g_ws) {
-            TL_HIP_TRY(hipStreamSynchronize(stream()));
-            TL_HIP_TRY(hipFree(g_ws));
-            g_ws = nullptr;
-            g_ws_floats = 0;
-        }
-        size_t want = floats < (1u << 20) ? (1u << 20) : floats;
-        hipError_t e = hipMalloc((void**)&g_ws, want * sizeof(float));
-        if (e != hipSuccess) {
-            (void)hipGetLastError();
-            return set_error(TL_ENOMEM, "attention workspace: hipMalloc(%zu bytes) failed: %s", want * sizeof(float),
-                             hipGetErrorString(e));
-        }
-        g_ws_floats = want;
-    }
-    *out = g_ws;
-    return TL_OK;
-}
+static Workspace g_partials;
 
 }  // namespace tl
 
@@ -875,11 +852,13 @@ static int launch_decode_attention(void* out, const void* q, void* cache_k, void
     TL_REQUIRE(n_heads <= 65535, "%s: too many heads", name);
     const int n_chunks = (T + tl::kAttnChunk - 1) / tl::kAttnChunk;
     TL_REQUIRE(n_chunks <= 65535, "%s: T=%d too long", name, T);
-    float* ws = nullptr;
+    tl::Workspace::Lease lease;   // held until both kernels are enqueued
     if (n_chunks > 1) {
-        int rc = tl::workspace((size_t)n_heads * n_chunks * (head_dim + 2), &ws);
+        int rc = tl::g_partials.acquire((size_t)n_heads * n_chunks * (head_dim + 2), (size_t)1 << 20,
+                                        "attention workspace", &lease);
         if (rc != TL_OK) return rc;
     }
+    float* ws = lease.ptr;
     // the reference divides the scores by half(sqrt(head_dim)) (Transformer.cpp:94)
     const float scale = (float)(tl::half_t)sqrtf((float)head_dim);
     const float inv_scale = 1.0f / scale;
@@ -1106,9 +1085,11 @@ int tl_hgemm_add_rms_norm_f16(const void* A, const void* W, const void* residual
                      tl::aligned16(residual) && tl::aligned16(norm_weight);
     float* slabs = nullptr;
     int splits = 1;
+    tl::Workspace::Lease lease;   // keeps the split-K slabs in place until the norm kernel that reads them is enqueued
     // the product goes to norm_out (overwritten by the normalised rows afterwards) unless K was split
     int rc = M == 1 ? tl::launch_gemv(A, W, norm_out, N, K, 1, 0, 0, 0, 0)
-                    : tl::launch_hgemm(A, W, norm_out, M, N, K, 1, 0, 0, 0, vec ? &slabs : nullptr, vec ? &splits : nullptr);
+                    : tl::launch_hgemm(A, W, norm_out, M, N, K, 1, 0, 0, 0, vec ? &slabs : nullptr, vec ? &splits : nullptr,
+                                       &lease);
     if (rc != TL_OK) return rc;
     if (splits <= 1) return tl_add_rms_norm_f16(sum_out, norm_out, residual, norm_out, norm_weight, eps, (int)N, (int)M);
     const int cpt = (int)((N / 8 + 511) / 512);

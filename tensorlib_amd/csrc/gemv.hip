@@ -11,6 +11,7 @@
 //     (used for the 11008-wide down-projection); partial sums meet in LDS, in a fixed order;
 //   * the 64 partial sums of a wavefront are combined with DPP row operations and
 //     four v_readlane, no LDS traffic.
+#include <atomic>
 #include <cstring>
 
 #include "tl_internal.h"
@@ -445,8 +446,8 @@ static const GemvVariant g_variants[] = {
 };
 
 static constexpr int kNumVariants = sizeof(g_variants) / sizeof(g_variants[0]);
-static int g_forced_variant = 0;
-static int g_grid_waves_per_cu = 0;  // 0 = automatic
+static std::atomic<int> g_forced_variant{0};
+static std::atomic<int> g_grid_waves_per_cu{0};  // 0 = automatic
 
 static int variant_index(const char* name) {
     for (int i = 0; i < (int)(sizeof(g_variants) / sizeof(g_variants[0])); ++i)
@@ -514,7 +515,8 @@ int launch_gemv(const void* x, const void* W, void* y, size_t N, size_t K, size_
     a.sum_out = norm ? (half8_t*)norm->sum_out : nullptr;
     a.eps = norm ? norm->eps : 0.f;
 
-    if (a.K8 < 64 && g_forced_variant == 0) {
+    const int forced_variant = g_forced_variant.load();
+    if (a.K8 < 64 && forced_variant == 0) {
         int lpr = a.K8 >= 32 ? 32 : a.K8 >= 16 ? 16 : 8;
         int rows_per_block = 4 * (64 / lpr);
         a.num_row_blocks = (int)((N + rows_per_block - 1) / rows_per_block);
@@ -533,7 +535,7 @@ int launch_gemv(const void* x, const void* W, void* y, size_t N, size_t K, size_
     }
 
     int auto_wpc = 16;
-    int vi = g_forced_variant ? g_forced_variant : pick_variant(N, K, &auto_wpc);
+    int vi = forced_variant ? forced_variant : pick_variant(N, K, &auto_wpc);
     if (prologue == 1) {
         static const int v_k4096 = variant_index("stream_w4r2u2s4x2");
         static const int v_k12288 = variant_index("stream_w8r2u3s8x2");
@@ -559,7 +561,7 @@ int launch_gemv(const void* x, const void* W, void* y, size_t N, size_t K, size_
         const GemvVariant& sv = g_variants[vi];
         const int seg = (a.K8 + sv.ksplit - 1) / sv.ksplit;
         if (seg > 64 * sv.unroll) {
-            TL_REQUIRE(g_forced_variant == 0, "gemv variant %s cannot hold K=%zu (segment %d chunks > %d)", sv.name, K,
+            TL_REQUIRE(forced_variant == 0, "gemv variant %s cannot hold K=%zu (segment %d chunks > %d)", sv.name, K,
                        seg, 64 * sv.unroll);
             vi = variant_index("loop_w4r2u6s4nttrue");
         }
@@ -583,7 +585,8 @@ int launch_gemv(const void* x, const void* W, void* y, size_t N, size_t K, size_
         return TL_OK;
     }
     int blocks = a.num_row_blocks;
-    int wpc = g_grid_waves_per_cu > 0 ? g_grid_waves_per_cu : auto_wpc;
+    const int forced_wpc = g_grid_waves_per_cu.load();
+    int wpc = forced_wpc > 0 ? forced_wpc : auto_wpc;
     long cap = (long)dev.cu_count * wpc / v.waves;
     if (cap < 1) cap = 1;
     if (blocks > cap) blocks = (int)cap;

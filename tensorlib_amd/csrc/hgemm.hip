@@ -16,6 +16,7 @@
 // three stages, is persistent over C tiles.  hgemm_f16_mfma_kernel (any K % 8 == 0) stages tiles through
 // registers into LDS rows of BK+8 halves (the 16-byte pad makes the 32 rows a ds_read_b128 touches fall
 // in distinct bank groups) and zero-fills the K tail.  gemm_generic_kernel covers everything else.
+#include <atomic>
 #include <cstring>
 #include <mutex>
 #include <numeric>
@@ -678,38 +679,16 @@ static const HgemmVariant g_variants[] = {
 };
 
 static constexpr int kNumVariants = sizeof(g_variants) / sizeof(g_variants[0]);
-static int g_forced_variant = 0;
-static bool g_attr_set[kNumVariants] = {false};
+// Tuning knobs (tests and sweeps set them, any thread may read them while launching).
+static std::atomic<int> g_forced_variant{0};
+static std::atomic<bool> g_attr_set[kNumVariants];
 
-static int g_forced_splits = 0;  // 0 = automatic
-static int g_forced_rot_tile = -1, g_forced_rot_xcd = -1;  // -1 = automatic
-static int g_forced_band = 0;                              // 0 = automatic
+static std::atomic<int> g_forced_splits{0};  // 0 = automatic
+static std::atomic<int> g_forced_rot_tile{-1}, g_forced_rot_xcd{-1};  // -1 = automatic
+static std::atomic<int> g_forced_band{0};                              // 0 = automatic
 
 // Library-owned fp32 workspace for split-K partial sums, grown on demand (stream-ordered reuse).
-static std::mutex g_ws_mu;
-static float* g_ws = nullptr;
-static size_t g_ws_floats = 0;
-static int hgemm_workspace(size_t floats, float** out) {
-    std::lock_guard<std::mutex> lk(g_ws_mu);
-    if (floats > g_ws_floats) {
-        if (g_ws) {
-            TL_HIP_TRY(hipStreamSynchronize(stream()));
-            TL_HIP_TRY(hipFree(g_ws));
-            g_ws = nullptr;
-            g_ws_floats = 0;
-        }
-        const size_t want = floats < (size_t)(8u << 20) ? (size_t)(8u << 20) : floats;
-        hipError_t e = hipMalloc((void**)&g_ws, want * sizeof(float));
-        if (e != hipSuccess) {
-            (void)hipGetLastError();
-            return set_error(TL_ENOMEM, "split-K workspace: hipMalloc(%zu bytes) failed: %s", want * sizeof(float),
-                             hipGetErrorString(e));
-        }
-        g_ws_floats = want;
-    }
-    *out = g_ws;
-    return TL_OK;
-}
+static Workspace g_splitk;
 
 static size_t lds_bytes(const HgemmVariant& v) {
     if (v.stages > 0) return (size_t)v.stages * (v.bm + v.bn) * v.bk * sizeof(half_t);
@@ -773,7 +752,9 @@ static int pick_variant(size_t M, size_t N, size_t K, int cus) {
 }
 
 int launch_hgemm(const void* A, const void* B, void* C, size_t M, size_t N, size_t K, size_t batch, size_t sa,
-                 size_t sb, size_t sc, float** partials_out, int* splits_out) {
+                 size_t sb, size_t sc, float** partials_out, int* splits_out, Workspace::Lease* lease_out) {
+    Workspace::Lease own_lease;
+    Workspace::Lease& lease = lease_out ? *lease_out : own_lease;
     if (splits_out) *splits_out = 1;
     if (M == 0 || N == 0 || batch == 0) return TL_OK;
     TL_REQUIRE(M <= 0x7fffffffu && N <= 0x7fffffffu && K <= 0x7fffffffu && batch <= 65535,
@@ -796,16 +777,17 @@ int launch_hgemm(const void* A, const void* B, void* C, size_t M, size_t N, size
         TL_CHECK_LAUNCH("gemm_generic_kernel<half>");
         return TL_OK;
     }
-    int vi = g_forced_variant ? g_forced_variant : pick_variant(M, N, K, device_info().cu_count);
+    const int forced_variant = g_forced_variant.load();
+    int vi = forced_variant ? forced_variant : pick_variant(M, N, K, device_info().cu_count);
     if (g_variants[vi].stages > 0 && K % g_variants[vi].bk != 0) vi = 1;  // direct-to-LDS path cannot zero-fill a K tail
     // its per-lane byte offsets inside a tile ((rows - 1) * K + 64 halves) are 32-bit
     if (g_variants[vi].stages > 0 && K > ((size_t)1 << 22)) vi = 1;
     const HgemmVariant& v = g_variants[vi];
     const size_t lds = lds_bytes(v);
-    if (lds > 64 * 1024 && !g_attr_set[vi]) {
+    if (lds > 64 * 1024 && !g_attr_set[vi].load()) {
         TL_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(v.kernel),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-        g_attr_set[vi] = true;
+        g_attr_set[vi].store(true);
     }
     HgemmArgs a;
     a.A = (const half_t*)A;
@@ -826,14 +808,15 @@ int launch_hgemm(const void* A, const void* B, void* C, size_t M, size_t N, size
     a.rot_tile = 0;
     a.rot_xcd = 0;
     // band height that balances the panels of A and B an XCD's 32 tiles pull through its L2
-    a.band_m = g_forced_band > 0 ? g_forced_band : (v.bm >= 2 * v.bn ? 4 : 8);
+    const int forced_band = g_forced_band.load();
+    a.band_m = forced_band > 0 ? forced_band : (v.bm >= 2 * v.bn ? 4 : 8);
     int splits = 1;
     if (v.stages > 0) {
         // Split K when the tile grid alone cannot occupy the chip (prefill with few tokens: the
         // problem is then bound by streaming W, and every CU has to pull on it).
         const int KT = (int)(K / v.bk);
         const int cus = device_info().cu_count;
-        splits = g_forced_splits;
+        splits = g_forced_splits.load();
         if (splits <= 0) {
             // aim at one workgroup per CU, keep at least 8 K tiles per split
             // (only for few rows: with more than 512 rows pick_variant already found a tile shape that
@@ -849,8 +832,9 @@ int launch_hgemm(const void* A, const void* B, void* C, size_t M, size_t N, size
         if (splits > 1) {
             a.kt_per_split = (KT + splits - 1) / splits;
             splits = (KT + a.kt_per_split - 1) / a.kt_per_split;
-            int rc = hgemm_workspace((size_t)splits * M * N, &a.partial);
+            int rc = g_splitk.acquire((size_t)splits * M * N, (size_t)8 << 20, "split-K workspace", &lease);
             if (rc != TL_OK) return rc;
+            a.partial = lease.ptr;
         }
     }
     // pipelined kernels with up to three stages are persistent: one workgroup per resident slot walks several tiles
@@ -869,8 +853,9 @@ int launch_hgemm(const void* A, const void* B, void* C, size_t M, size_t N, size
         } else {
             a.rot_xcd = kt_walk / 8;  // tiles of one XCD keep walking K together (they share panels through its L2)
         }
-        if (g_forced_rot_tile >= 0) a.rot_tile = g_forced_rot_tile;
-        if (g_forced_rot_xcd >= 0) a.rot_xcd = g_forced_rot_xcd;
+        const int rt = g_forced_rot_tile.load(), rx = g_forced_rot_xcd.load();
+        if (rt >= 0) a.rot_tile = rt;
+        if (rx >= 0) a.rot_xcd = rx;
     }
     hipLaunchKernelGGL(v.kernel, dim3((unsigned)grid_x, (unsigned)batch, (unsigned)splits), dim3(v.threads), lds, st, a);
     TL_CHECK_LAUNCH(v.name);

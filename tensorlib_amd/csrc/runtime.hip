@@ -1,6 +1,7 @@
 // Runtime half of the C ABI: device selection, stream, memory, copies, error text.
 // Counterpart of the allocation / memcpy / error-check plumbing in the reference's
 // tensorLib/src/device/cuda/CUDA.cu:16-32,71-81 and tensorLib/include/device/cuda/CUDA.cuh:131-151.
+#include <atomic>
 #include <cstring>
 #include <mutex>
 
@@ -21,7 +22,7 @@ void clear_error() { g_err[0] = 0; }
 
 static std::mutex g_mu;
 static DeviceInfo g_info;
-static bool g_ready = false;
+static std::atomic<bool> g_ready{false};
 static hipStream_t g_stream = nullptr;
 
 hipStream_t stream() { return g_stream; }
@@ -45,17 +46,43 @@ static int init_locked(int ordinal) {
     if (strncmp(g_info.arch, "gfx950", 6) != 0)
         return set_error(TL_EHIP, "this library is built for gfx950 only, device %d is %s", ordinal,
                          g_info.arch);
-    g_ready = true;
+    g_ready.store(true, std::memory_order_release);
     return TL_OK;
 }
 
 int ensure_init() {
-    if (g_ready) return TL_OK;
+    if (g_ready.load(std::memory_order_acquire)) return TL_OK;
     std::lock_guard<std::mutex> lk(g_mu);
-    if (g_ready) return TL_OK;
+    if (g_ready.load(std::memory_order_relaxed)) return TL_OK;
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess) dev = 0;
     return init_locked(dev);
+}
+
+int Workspace::acquire(size_t floats, size_t min_floats, const char* what, Lease* lease) {
+    lease->lock = std::unique_lock<std::mutex>(mu_);
+    hipStream_t st = stream();
+    if (used_ && st != last_stream_) TL_HIP_TRY(hipStreamSynchronize(last_stream_));
+    if (floats > floats_) {
+        if (ptr_) {
+            TL_HIP_TRY(hipStreamSynchronize(st));
+            TL_HIP_TRY(hipFree(ptr_));
+            ptr_ = nullptr;
+            floats_ = 0;
+        }
+        const size_t want = floats < min_floats ? min_floats : floats;
+        hipError_t e = hipMalloc((void**)&ptr_, want * sizeof(float));
+        if (e != hipSuccess) {
+            (void)hipGetLastError();
+            return set_error(TL_ENOMEM, "%s: hipMalloc(%zu bytes) failed: %s", what, want * sizeof(float),
+                             hipGetErrorString(e));
+        }
+        floats_ = want;
+    }
+    last_stream_ = st;
+    used_ = true;
+    lease->ptr = ptr_;
+    return TL_OK;
 }
 
 }  // namespace tl
@@ -64,7 +91,7 @@ extern "C" {
 
 int tl_init(int device_ordinal) {
     std::lock_guard<std::mutex> lk(tl::g_mu);
-    if (tl::g_ready && tl::g_info.ordinal == device_ordinal) return TL_OK;
+    if (tl::g_ready.load(std::memory_order_acquire) && tl::g_info.ordinal == device_ordinal) return TL_OK;
     return tl::init_locked(device_ordinal);
 }
 
@@ -72,7 +99,7 @@ const char* tl_last_error(void) { return tl::g_err; }
 
 const char* tl_version(void) { return "tensorlib_amd 0.1 gfx950"; }
 
-int tl_device_cu_count(void) { return tl::g_ready ? tl::g_info.cu_count : 0; }
+int tl_device_cu_count(void) { return tl::g_ready.load(std::memory_order_acquire) ? tl::g_info.cu_count : 0; }
 
 int tl_set_stream(void* hip_stream) {
     tl::g_stream = static_cast<hipStream_t>(hip_stream);

@@ -5,6 +5,7 @@
 #include <cstddef>
 #include <cstdint>
 #include <cstdio>
+#include <mutex>
 
 #include "tensorlib_amd.h"
 
@@ -37,6 +38,27 @@ struct DeviceInfo {
 const DeviceInfo& device_info();
 int ensure_init();
 
+// Library-owned fp32 device scratch that grows on demand (split-K partial sums, attention chunk partials).
+// acquire() returns with the buffer's mutex held by the lease: the caller keeps the lease alive until every
+// kernel that touches the pointer is enqueued, so no other host thread can grow (free) the buffer in between.
+// Reuse is ordered by the stream: when the library's stream changed since the last user, that stream is drained
+// first.
+class Workspace {
+ public:
+    struct Lease {
+        std::unique_lock<std::mutex> lock;
+        float* ptr = nullptr;
+    };
+    int acquire(size_t floats, size_t min_floats, const char* what, Lease* lease);
+
+ private:
+    std::mutex mu_;
+    float* ptr_ = nullptr;
+    size_t floats_ = 0;
+    hipStream_t last_stream_ = nullptr;
+    bool used_ = false;
+};
+
 // out[i] = bits for i < n, as a kernel (safe to record into a HIP graph).
 int launch_fill_f16(void* out, uint16_t bits, size_t n);
 
@@ -54,8 +76,10 @@ int launch_gemv(const void* x, const void* W, void* y, size_t N, size_t K, size_
 // partials_out / splits_out (both or neither): when K was split, the fp32 slabs [splits][M][N] are handed to the
 // caller instead of being reduced into C (library-owned, valid until the next GEMM on the stream); *splits_out == 1
 // means C holds the result.
+// `lease` then keeps the slabs' buffer locked until the caller has enqueued its consumer.
 int launch_hgemm(const void* A, const void* B, void* C, size_t M, size_t N, size_t K, size_t batch,
-                 size_t sa, size_t sb, size_t sc, float** partials_out = nullptr, int* splits_out = nullptr);
+                 size_t sa, size_t sb, size_t sc, float** partials_out = nullptr, int* splits_out = nullptr,
+                 Workspace::Lease* lease = nullptr);
 
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
