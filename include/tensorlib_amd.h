@@ -219,6 +219,19 @@ int tl_hgemm_add_rms_norm_f16(const void* A, const void* W, const void* residual
 int tl_decode_attention_rope_f16(void* out, const void* qkv, void* cache_k, void* cache_v,
                                  const void* rope_table, int pos, int n_heads, int head_dim);
 
+/* tl_decode_attention_rope_f16 for callers that cannot allocate (code under HIP-graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc).  It has no counterpart in the reference.  Same kernels, same arguments, same
+ * results; the per-chunk partial results go to a static device array of TL_DECODE_ATTENTION_STATIC_SCRATCH_FLOATS
+ * floats that is part of the library's code object (each GPU holds its copy until the process ends) instead of the
+ * grown-on-demand workspace, and the call makes no hipMalloc / hipFree.  Limit:
+ *   n_heads * ceil((pos + 1) / 64) * (head_dim + 2) <= TL_DECODE_ATTENTION_STATIC_SCRATCH_FLOATS
+ * (32 heads of 128: 16128 positions); larger sizes return TL_EINVAL.  Every call on a GPU shares that GPU's array:
+ * calls that overlap on one GPU (two streams, two host threads) race; calls on one stream do not.  Nothing in the
+ * array has to start at zero (every slot a call reads was written by the same call). */
+#define TL_DECODE_ATTENTION_STATIC_SCRATCH_FLOATS (1u << 20)
+int tl_decode_attention_rope_static_f16(void* out, const void* qkv, void* cache_k, void* cache_v,
+                                        const void* rope_table, int pos, int n_heads, int head_dim);
+
 /* table[pos][pair] = (half(cos), half(sin)) of pos / 10000^(2*pair/head_dim) for pos < max_seq:
  * max_seq * head_dim halves.  The same values every RoPE entry point computes on the fly
  * (tensorLib/src/device/cpu/CPU.cpp:444-447); the reference's own precompute_freqs table is unused

@@ -91,6 +91,7 @@ _PROTOS = {
     "tl_gemv_add_rms_norm_f16": (_i, [_vp, _vp, _vp, _f, _vp, _vp, _vp, _sz, _sz]),
     "tl_hgemm_add_rms_norm_f16": (_i, [_vp, _vp, _vp, _vp, _f, _vp, _vp, _sz, _sz, _sz]),
     "tl_decode_attention_rope_f16": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i]),
+    "tl_decode_attention_rope_static_f16": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i]),
     "tl_rope_table_f16": (_i, [_vp, _i, _i]),
     "tl_rope_qk_store_kv_f16": (_i, [_vp, _vp, _vp, _i, _i, _i]),
     "tl_add_rms_norm_f16": (_i, [_vp, _vp, _vp, _vp, _vp, _f, _i, _i]),

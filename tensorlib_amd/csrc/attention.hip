@@ -838,10 +838,44 @@ static Workspace g_partials;
 
 }  // namespace tl
 
+// Chunk partials of tl_decode_attention_rope_static_f16, the entry point that allocates nothing: the memory is part
+// of the code object, so every GPU the library runs on holds its own copy from load time until the process ends.
+// `scratch` is a host-side stand-in for the symbol, not a device address: host code only ever passes the pointer
+// hipGetSymbolAddress returned for the current device.
+static __device__ __align__(256) float scratch[TL_DECODE_ATTENTION_STATIC_SCRATCH_FLOATS];
+
+namespace tl {
+
+constexpr int kMaxDevices = 64;
+static std::mutex g_scratch_mu;
+static float* g_scratch_ptr[kMaxDevices] = {nullptr};   // device address of `scratch`, per device ordinal
+
+// Resolves the current device's copy of `scratch` (once per device; called from the library's init and, for a
+// device the library was not initialised on, from the entry point's first call there).
+int attention_static_scratch(float** out) {
+    int dev = -1;
+    TL_HIP_TRY(hipGetDevice(&dev));
+    TL_REQUIRE(dev >= 0 && dev < kMaxDevices, "static attention scratch: device ordinal %d not supported", dev);
+    std::lock_guard<std::mutex> lk(g_scratch_mu);
+    if (!g_scratch_ptr[dev]) {
+        float* p = nullptr;
+        TL_HIP_TRY(hipGetSymbolAddress((void**)&p, HIP_SYMBOL(scratch)));
+        TL_REQUIRE(p != nullptr, "static attention scratch: hipGetSymbolAddress returned a null address");
+        g_scratch_ptr[dev] = p;
+    }
+    if (out) *out = g_scratch_ptr[dev];
+    return TL_OK;
+}
+
+}  // namespace tl
+
 extern "C" {
 
+// static_ws: null = partials go to the library's grown-on-demand workspace; else the caller's buffer of
+// static_ws_floats floats (no allocation on this path).
 static int launch_decode_attention(void* out, const void* q, void* cache_k, void* cache_v, const void* rope_table,
-                                   int T, int n_heads, int head_dim, bool fuse_rope, const char* name) {
+                                   int T, int n_heads, int head_dim, bool fuse_rope, const char* name,
+                                   float* static_ws = nullptr, size_t static_ws_floats = 0) {
     TL_ENSURE_INIT();
     TL_REQUIRE(out && q && cache_k && cache_v, "%s: null pointer", name);
     TL_REQUIRE(T >= 1 && n_heads >= 1, "%s: bad sizes T=%d n_heads=%d", name, T, n_heads);
@@ -853,12 +887,18 @@ static int launch_decode_attention(void* out, const void* q, void* cache_k, void
     const int n_chunks = (T + tl::kAttnChunk - 1) / tl::kAttnChunk;
     TL_REQUIRE(n_chunks <= 65535, "%s: T=%d too long", name, T);
     tl::Workspace::Lease lease;   // held until both kernels are enqueued
-    if (n_chunks > 1) {
-        int rc = tl::g_partials.acquire((size_t)n_heads * n_chunks * (head_dim + 2), (size_t)1 << 20,
-                                        "attention workspace", &lease);
+    const size_t ws_floats = (size_t)n_heads * n_chunks * (head_dim + 2);
+    float* ws = static_ws;
+    if (static_ws) {
+        TL_REQUIRE(ws_floats <= static_ws_floats,
+                   "%s: %d heads x %d chunks of 64 positions x (%d + 2) floats = %zu floats of partial results exceed the "
+                   "static scratch of %zu floats; use tl_decode_attention_rope_f16 for this size",
+                   name, n_heads, n_chunks, head_dim, ws_floats, static_ws_floats);
+    } else if (n_chunks > 1) {
+        int rc = tl::g_partials.acquire(ws_floats, (size_t)1 << 20, "attention workspace", &lease);
         if (rc != TL_OK) return rc;
+        ws = lease.ptr;
     }
-    float* ws = lease.ptr;
     // the reference divides the scores by half(sqrt(head_dim)) (Transformer.cpp:94)
     const float scale = (float)(tl::half_t)sqrtf((float)head_dim);
     const float inv_scale = 1.0f / scale;
@@ -903,6 +943,19 @@ int tl_decode_attention_rope_f16(void* out, const void* qkv, void* cache_k, void
     TL_REQUIRE(rope_table == nullptr || tl::aligned16(rope_table), "tl_decode_attention_rope_f16: misaligned table");
     return launch_decode_attention(out, qkv, cache_k, cache_v, rope_table, pos + 1, n_heads, head_dim, true,
                                    "tl_decode_attention_rope_f16");
+}
+
+int tl_decode_attention_rope_static_f16(void* out, const void* qkv, void* cache_k, void* cache_v, const void* rope_table,
+                                        int pos, int n_heads, int head_dim) {
+    TL_ENSURE_INIT();
+    TL_REQUIRE(pos >= 0, "tl_decode_attention_rope_static_f16: negative position");
+    TL_REQUIRE(rope_table == nullptr || tl::aligned16(rope_table), "tl_decode_attention_rope_static_f16: misaligned table");
+    float* ws = nullptr;
+    int rc = tl::attention_static_scratch(&ws);   // a table lookup after the first call on a device
+    if (rc != TL_OK) return rc;
+    return launch_decode_attention(out, qkv, cache_k, cache_v, rope_table, pos + 1, n_heads, head_dim, true,
+                                   "tl_decode_attention_rope_static_f16", ws,
+                                   (size_t)TL_DECODE_ATTENTION_STATIC_SCRATCH_FLOATS);
 }
 
 int tl_rope_table_f16(void* table, int max_seq, int head_dim) {

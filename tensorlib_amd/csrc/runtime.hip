@@ -46,6 +46,10 @@ static int init_locked(int ordinal) {
     if (strncmp(g_info.arch, "gfx950", 6) != 0)
         return set_error(TL_EHIP, "this library is built for gfx950 only, device %d is %s", ordinal,
                          g_info.arch);
+    // resolve the static scratch of the entry point that allocates nothing now, with this device current,
+    // so that entry point itself only reads a table
+    int rc = attention_static_scratch(nullptr);
+    if (rc != TL_OK) return rc;
     g_ready.store(true, std::memory_order_release);
     return TL_OK;
 }

@@ -59,6 +59,10 @@ class Workspace {
     bool used_ = false;
 };
 
+// Looks up (once per device) the device address of the static scratch array behind
+// tl_decode_attention_rope_static_f16 for the current device; `out` may be null.
+int attention_static_scratch(float** out);
+
 // out[i] = bits for i < n, as a kernel (safe to record into a HIP graph).
 int launch_fill_f16(void* out, uint16_t bits, size_t n);
 

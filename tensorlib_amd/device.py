@@ -298,16 +298,22 @@ class HipDevice:
         return t
 
     def decode_attention_rope(self, qkv: torch.Tensor, cache_k: torch.Tensor, cache_v: torch.Tensor, pos: int,
-                              rope_table: torch.Tensor | None = None):
-        """qkv: [3, n_heads, head_dim] raw projections of the token at `pos`; writes cache rows `pos`."""
+                              rope_table: torch.Tensor | None = None, out: torch.Tensor | None = None,
+                              static_scratch: bool = False):
+        """qkv: [3, n_heads, head_dim] raw projections of the token at `pos`; writes cache rows `pos`.
+        static_scratch: go through the entry point that allocates nothing (then pass `out` too)."""
         _req(qkv, name="qkv"), _req(cache_k, name="cache_k"), _req(cache_v, name="cache_v")
         _, H, D = qkv.shape
         if cache_k.shape[1:] != (H, D) or cache_v.shape != cache_k.shape or pos >= cache_k.shape[0]:
             raise ValueError("cache shape does not match qkv / pos")
-        out = self.empty(H, D)
+        out = self.empty(H, D) if out is None else _req(out, name="out")
         tab = ctypes.c_void_p(0) if rope_table is None else _ptr(_req(rope_table, name="rope_table"))
-        check(self.lib.tl_decode_attention_rope_f16(_ptr(out), _ptr(qkv), _ptr(cache_k), _ptr(cache_v), tab, pos, H, D),
-              "tl_decode_attention_rope_f16")
+        if static_scratch:
+            check(self.lib.tl_decode_attention_rope_static_f16(_ptr(out), _ptr(qkv), _ptr(cache_k), _ptr(cache_v), tab,
+                                                               pos, H, D), "tl_decode_attention_rope_static_f16")
+        else:
+            check(self.lib.tl_decode_attention_rope_f16(_ptr(out), _ptr(qkv), _ptr(cache_k), _ptr(cache_v), tab, pos, H, D),
+                  "tl_decode_attention_rope_f16")
         return out
 
     def rope_qk_store_kv(self, qkv: torch.Tensor, cache_k: torch.Tensor, cache_v: torch.Tensor, pos: int):
