@@ -155,7 +155,16 @@ class HipDevice:
         boundary wants; for a Linear weight passed as ``W.t()`` no copy is made."""
         if a.device != b.device:
             raise ValueError("Tensors must be on the same device.")
+        for t, name in ((a, "a"), (b, "b")):          # strided views are fine here, dtype and device are not negotiable
+            if not isinstance(t, torch.Tensor) or not t.is_cuda:
+                raise TensorLibError(f"{name} must be a CUDA(HIP) tensor; there is no CPU path")
+            if t.dtype != torch.float16:
+                raise TypeError(f"{name} must be torch.float16, got {t.dtype}")
         ab, bb, obatch, M, N, K = plan_matmul(a.shape, b.shape, None if out is None else out.shape)
+        # The temporaries below return to torch's caching allocator while the kernel may still be queued: that is
+        # safe only because the library enqueues on the stream torch considers current, which is checked here.
+        if (self.lib.tl_get_stream() or 0) != torch.cuda.current_stream().cuda_stream:
+            raise TensorLibError("the library stream is not torch's current stream; call bind_stream(torch.cuda.current_stream()) first")
         A = a.contiguous()
         Bt = b.transpose(-2, -1).contiguous()  # [..., N, K]; a view of a Linear weight stays a view
         oshape = obatch + [M, N]

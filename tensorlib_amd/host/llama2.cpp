@@ -78,6 +78,18 @@ struct tlm_model {
     std::vector<Buf> cache_k, cache_v;  // per layer [max_seq, n_heads, head_dim]
     Buf x, x_norm, x_residual, qkv, x13, x2, scores, scores2, mask, xq_c, keys_c, values_c, s_v, o_c, logits;
     Buf rope_table;  // [max_seq][head_dim/2][cos, sin], filled once at creation
+
+    // Score matrices, mask and gathered keys (n_heads * max_tokens * max_seq halves each, ~0.8 GB at 32 heads with
+    // 2048 x 2048) serve only the reference op chain and head sizes the fused attention does not cover: they are
+    // allocated when such a forward first runs.
+    void need_chain_buffers() {
+        if (scores.p) return;
+        const size_t sc = (size_t)n_heads * max_tokens * max_seq;
+        scores.alloc(sc);
+        scores2.alloc(sc);
+        mask.alloc(sc);
+        keys_c.alloc((size_t)max_seq * dim);
+    }
     std::vector<void*> owned_weights;  // device allocations made by tlm_load_checkpoint
     int* d_tokens = nullptr;   // [max_tokens + generated]
     int d_tokens_cap = 0;
@@ -305,6 +317,7 @@ struct tlm_model {
                 ck(tl_prefill_attention_f16(o_c.p, xq_c.p, cache_k[l].p, values_c.p, ldv, start_pos, S, H, D),
                    "prefill_attention");
             } else {
+            need_chain_buffers();
             // keys -> [H,T,D], values -> [H,D,T] (what the per-head matmul2d calls consume)   Transformer.cpp:61-80
             cache_k[l].dev->contiguous(keys_c.p, {1, H, T, D}, {max_seq * dim, D, dim, 1}, 0, (size_t)T * dim);
             cache_v[l].dev->contiguous(values_c.p, {1, H, D, T}, {max_seq * dim, D, 1, dim}, 0, (size_t)T * dim);
@@ -354,6 +367,7 @@ struct tlm_model {
             }
             return logits.p;
         }
+        need_chain_buffers();
         const bool use_mask = S > 1;   // get_mask: nullopt when seqlen <= 1   Transformer.cpp:234
         if (use_mask) ck(tl_causal_mask_f16(mask.p, n_heads, S, start_pos), "causal_mask");
         for (int l = 0; l < n_layers; ++l) block_chain(l, S, start_pos, use_mask);
@@ -398,10 +412,7 @@ int tlm_create(tlm_model** out, int dim, int hidden_dim, int n_layers, int n_hea
         m->qkv.alloc(3 * sd);
         m->x13.alloc(2 * S * hidden_dim);
         m->x2.alloc(S * hidden_dim);
-        const size_t sc = (size_t)n_heads * S * max_seq_len;
-        m->scores.alloc(sc); m->scores2.alloc(sc); m->mask.alloc(sc);
         m->xq_c.alloc(sd); m->s_v.alloc(sd); m->o_c.alloc(sd);
-        m->keys_c.alloc((size_t)max_seq_len * dim);
         m->values_c.alloc((size_t)((max_seq_len + 63) / 64 * 64) * dim);   // rows padded for the prefill attention
         m->logits.alloc(S * vocab_size);
         m->rope_table.alloc((size_t)max_seq_len * (dim / n_heads));

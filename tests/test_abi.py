@@ -4,6 +4,9 @@ product package never reaches into the oracle.  No compute call is made here."""
 import ctypes
 import os
 import re
+import subprocess
+
+import pytest
 
 from tensorlib_amd import _lib
 
@@ -80,3 +83,29 @@ def test_product_never_imports_the_oracle():
             if f.endswith((".py", ".hip", ".h", ".hpp", ".cpp", "Makefile")):
                 src = open(os.path.join(dirpath, f), errors="ignore").read()
                 assert "oracle" not in src.lower(), os.path.join(dirpath, f)
+
+
+REFERENCE_INCLUDE = "/root/reference/tensorLib/include"
+
+
+@pytest.mark.skipif(not os.path.exists(os.path.join(REFERENCE_INCLUDE, "device", "Device.hpp")),
+                    reason="the reference tree is not present (it never is on the GPU box)")
+def test_adaptor_overrides_every_pure_virtual_of_the_reference_interface(tmp_path):
+    """include/tl_hip_device.hpp compiled against the reference's own Device.hpp
+    (tensorLib/include/device/Device.hpp:13-101): deriving from Device<dtype> with every method marked
+    `override`, and instantiating HIP<half>, HIP<int> and HIP<float>, only compiles when each pure virtual is
+    overridden with a matching signature.  Syntax check only: nothing is linked or run."""
+    src = tmp_path / "adaptor_check.cpp"
+    src.write_text(
+        '#include "tl_hip_device.hpp"\n'
+        "template class HIP<tl::half>;\n"
+        "template class HIP<int>;\n"
+        "template class HIP<float>;\n"
+        "Device<tl::half>* make_h(size_t n) { return new HIP<tl::half>(n); }\n"
+        "Device<int>* make_i(size_t n) { return new HIP<int>(n); }\n"
+        "Device<float>* make_f(size_t n) { return new HIP<float>(n); }\n")
+    cxx = "/opt/rocm/lib/llvm/bin/clang++"      # needs _Float16 on the host, which g++ 11 lacks
+    proc = subprocess.run([cxx, "-std=c++17", "-fsyntax-only", "-Wall", "-Werror=overloaded-virtual",
+                           "-DTL_HAVE_TENSORLIB_DEVICE_HPP", "-I", os.path.join(ROOT, "include"), "-I", REFERENCE_INCLUDE,
+                           str(src)], capture_output=True, text=True)
+    assert proc.returncode == 0, proc.stderr[-3000:]
