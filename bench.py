@@ -42,7 +42,10 @@ HGEMM_SHAPES = [(2048, 4096, 4096), (2048, 11008, 4096), (2048, 32000, 4096), (2
 # HBM bytes per GEMV launch measured with rocprofv3 --pmc (FETCH_SIZE, WRITE_SIZE), averaged over
 # the four sweep launches and scaled by the same counters' reading for a copy kernel of known
 # size (FETCH_SIZE x 1.9997 KiB, WRITE_SIZE x 1.0000 KiB); algorithmic bytes per launch are 119,050,624.
-GEMV_TRAFFIC_BYTES_PER_LAUNCH = 119_423_152  # profiles/gemv_decode_sweep_hbm_traffic.txt
+# Counters cannot be read inside this process: the figure comes from the profile named beside it and is
+# reported with that source, not re-measured by a bench run.
+GEMV_TRAFFIC_BYTES_PER_LAUNCH = 119_423_152
+GEMV_TRAFFIC_SOURCE = "profiles/gemv_decode_sweep_hbm_traffic.txt (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of this command)"
 
 
 def parse_args():
@@ -110,6 +113,48 @@ def cpu_baseline_hgemm():
         "sample": f"{rows} rows of X of the 2048x4096x4096 shape ({rows}x{N}x{K}), median of 7 runs, "
                   f"{med * 1e3:.1f} ms; full shape would take {med * 2048 / rows:.2f} s (extrapolated)",
     }
+
+
+def cpu_baseline_llama2_decode(k: int = 6):
+    """Time k single-token decode steps of the CPU oracle's Llama2 op chain at Llama2-7B size (32 layers of
+    dim 4096 / hidden 11008 / 32 heads, vocabulary 32000, context 128..128+k).  Bounded sample: the 32 layers
+    cycle over two distinct random-init weight sets (2 x 405 MB, far beyond the host caches, so every GEMV still
+    streams its matrix from memory as 32 distinct layers would) instead of 13 GB drawn fresh; the embedding table
+    shares the classifier's array.  Arithmetic per step is exactly that of the full model."""
+    import numpy as np
+    from oracle import oracle
+    from oracle.llama2_oracle import Llama2Oracle
+    from tensorlib_amd import synth
+    dim, hidden, L, H, vocab = 4096, 11008, 32, 32, 32000
+    w = {"classifier": synth.normal_f16(900, (vocab, dim), 0.02), "final_norm": synth.normal_f16(901, (dim,), 1.0)}
+    w["tok_emb"] = w["classifier"]
+    distinct = 2
+    for s in range(distinct):
+        base = {"att_norm": synth.normal_f16(910 + 20 * s, (dim,), 1.0), "ffn_norm": synth.normal_f16(911 + 20 * s, (dim,), 1.0)}
+        for i, n in enumerate(("wq", "wk", "wv", "wo")):
+            base[n] = synth.normal_f16(912 + 20 * s + i, (dim, dim), 0.02)
+        base["w1"] = synth.normal_f16(916 + 20 * s, (hidden, dim), 0.02)
+        base["w3"] = synth.normal_f16(917 + 20 * s, (hidden, dim), 0.02)
+        base["w2"] = synth.normal_f16(918 + 20 * s, (dim, hidden), 0.02)
+        for l in range(s, L, distinct):
+            for n, a in base.items():
+                w[f"{n}.{l}"] = a
+    start = 128
+    m = Llama2Oracle(w, dim, hidden, L, H, vocab, start + k + 1, 1e-5)
+    for l in range(L):   # a context of 128 positions already in the cache
+        m.cache_k[l][:start] = synth.normal_f16(950, (start, H, dim // H), 1.0)
+        m.cache_v[l][:start] = synth.normal_f16(951, (start, H, dim // H), 1.0)
+    toks = synth.token_ids(960, k + 1, vocab)
+    m.forward(toks[:1], start)   # warm-up step (thread pool, page faults)
+    times = []
+    for i in range(k):
+        t0 = time.perf_counter()
+        m.forward(toks[i + 1:i + 2], start + 1 + i)
+        times.append(time.perf_counter() - t0)
+    med = float(np.median(times))
+    return {"value": round(1.0 / med, 3), "unit": "tok/s", "cores": oracle.max_threads(), "kind": "port",
+            "sample": f"{k} teacher-forced single-token steps of the oracle's op chain at Llama2-7B size, context 129..{start + k}, "
+                      f"layers cycling over {distinct} distinct weight sets; median {med * 1e3:.0f} ms per token"}
 
 
 def time_region(fn, reps: int, torch):
@@ -282,6 +327,7 @@ def main():
             "unit": "GB/s",
             "frac": round(achieved / HBM_PEAK_GBS, 4),
             "traffic": GEMV_TRAFFIC_BYTES_PER_LAUNCH,
+            "traffic_source": GEMV_TRAFFIC_SOURCE,
             "kernel": "gemv_f16_stream_kernel",
             "bytes_per_launch": step_bytes / len(SWEEP),
             "avg_launch_us": round(avg_launch_s * 1e6, 3),
@@ -293,7 +339,7 @@ def main():
     extra = {}
     if not args.no_extra:
         # per-shape GEMV, each over >1 GB of rotating weights
-        per_shape = {}
+        per_shape, cache_resident = {}, {}
         for (N, K) in SWEEP:
             nbuf = max(2, int(1.0e9 // (N * K * 2)) + 1)
             Ws = [randn((N, K), 0.02) for _ in range(nbuf)]
@@ -310,8 +356,25 @@ def main():
             us = ev1 / 200 * 1e6
             gbs = synth.gemv_bytes(N, K) / us / 1e3
             per_shape[f"{N}x{K}"] = {"us": round(us, 2), "GB/s": round(gbs, 1), "frac_hbm": round(gbs / HBM_PEAK_GBS, 4)}
+            # the same launch with ONE matrix used again and again: the three smaller ones then sit in the 256 MB
+            # memory-side cache, so this is the cache-resident figure, not an HBM figure
+            for _ in range(10):
+                dev.matmul2d(x, Ws[0], y)
+            _, ev2 = time_region(lambda: dev.matmul2d(x, Ws[0], y), 200, torch)
+            us2 = ev2 / 200 * 1e6
+            cache_resident[f"{N}x{K}"] = {"us": round(us2, 2), "GB/s": round(synth.gemv_bytes(N, K) / us2 / 1e3, 1)}
             del Ws
         extra["gemv_per_shape"] = per_shape
+        extra["gemv_cache_resident"] = cache_resident
+        # one decoded token launches 128 / 64 / 32 / 1 of the four shapes (wq wk wv wo / w1 w3 / w2 / classifier):
+        # the sweep's equal weights flatter the mix, this figure does not
+        mix = {(4096, 4096): 128, (11008, 4096): 64, (4096, 11008): 32, (32000, 4096): 1}
+        mix_bytes = sum(n * synth.gemv_bytes(N, K) for (N, K), n in mix.items())
+        mix_us = sum(n * per_shape[f"{N}x{K}"]["us"] for (N, K), n in mix.items())
+        extra["gemv_decode_mix"] = {"launches_per_token": {f"{N}x{K}": n for (N, K), n in mix.items()},
+                                    "bytes_per_token": mix_bytes, "us_per_token": round(mix_us, 1),
+                                    "GB/s": round(mix_bytes / mix_us / 1e3, 1),
+                                    "frac_hbm": round(mix_bytes / mix_us / 1e3 / HBM_PEAK_GBS, 4)}
         torch.cuda.empty_cache()
 
         sustained = mfma_sustained(dev)
@@ -324,6 +387,10 @@ def main():
 
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline_gemv()
+        if not args.no_extra:
+            # the other two metrics' CPU figures, on the same host in the same run
+            extra["hgemm_cpu_baseline"] = cpu_baseline_hgemm()
+            extra["llama2_7b_decode"]["cpu"] = cpu_baseline_llama2_decode()
     print(json.dumps(out))
 
 

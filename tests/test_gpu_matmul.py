@@ -135,6 +135,37 @@ def test_hgemm_prefill_shapes_sampled(dev, oracle, M, N, K):
     _hgemm_case(dev, oracle, M, N, K, seed=900 + M + N % 31, full=False)
 
 
+@pytest.mark.parametrize("M", [512, 2048])
+@pytest.mark.parametrize("N,K", [(4096, 4096), (11008, 4096), (32000, 4096), (4096, 11008)])
+def test_hgemm_prefill_whole_matrix_against_second_gpu_path(dev, oracle, M, N, K):
+    """Every entry of the large prefill products, not a sample.  The checker is the library's plain fp32 kernel
+    (tl_matmul2d_f32 on the operands widened to fp32: one thread per entry, one fp32 accumulator, k ascending),
+    which shares nothing with the MFMA kernels.  Products of two halves are exact in fp32, so that kernel's sum is
+    the CPU loop's sum (CPU.cpp:76-89) and its fp16 rounding must equal the oracle bit for bit, which is asserted
+    on eight rows.  The MFMA result may differ from it by the fp32 summation order only: the two fp32 sums differ
+    by rounding noise of the partial sums (magnitude ~1, K terms: a few 1e-6, bounded here by 2e-5), which after
+    the fp16 rounding is at most one fp16 ulp on top of that noise, and inside the parity gate everywhere."""
+    A = synth.normal_f16(2000 + M, (M, K), 1.0)
+    B = synth.normal_f16(2001 + N % 97, (N, K), 0.02)
+    Ad, Bd = dev.from_numpy(A), dev.from_numpy(B)
+    ref = dev.matmul2d_f32(Ad.float(), Bd.float()).half()
+    rng = np.random.default_rng(M + N)
+    rows = np.unique(np.concatenate([[0, M - 1], rng.integers(0, M, 6)]))
+    want = oracle.matmul2d(A[rows], B)
+    assert np.array_equal(ref[torch.as_tensor(rows, device=ref.device)].cpu().numpy().view(np.uint16), want.view(np.uint16)), \
+        "the fp32 checker kernel does not reproduce the CPU loop"
+    C = dev.hgemm(Ad, Bd)
+    cf, rf = C.float(), ref.float()
+    err = (cf - rf).abs()
+    # spacing of fp16 at the larger of the two magnitudes (2^-24 below the smallest normal): x = m * 2^e with
+    # m in [0.5, 1) has spacing 2^(e - 11)
+    _, e = torch.frexp(torch.maximum(cf.abs(), rf.abs()).clamp_min(2.0 ** -14))
+    ulp = torch.pow(2.0, (e - 11).float())
+    assert bool((err <= ulp + 2e-5).all()), f"{int((err > ulp + 2e-5).sum())} entries differ by more than one fp16 ulp"
+    assert bool((err <= ATOL + RTOL * rf.abs()).all()), "whole-matrix parity gate"
+    assert float((err > 0).float().mean()) < 0.2, "an unexpected share of entries rounds differently"
+
+
 def test_hgemm_every_variant_ragged(dev, oracle):
     names = dev.hgemm_variants()
     for v in range(1, len(names)):
