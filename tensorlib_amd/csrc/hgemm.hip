@@ -31,6 +31,7 @@ struct HgemmArgs {
     const half_t* B;
     half_t* C;
     int M, N, K;
+    int ldc;  // elements between rows of C (N, unless the launch covers a column range of a wider C)
     int tiles_m, tiles_n;
     long sa, sb, sc;  // batch strides in elements
     // split-K (direct-to-LDS kernel only): blockIdx.z walks K tiles [z*kt_per_split, ...) and writes
@@ -197,7 +198,7 @@ __global__ void __launch_bounds__(WM* WN * 64) hgemm_f16_mfma_kernel(HgemmArgs a
 #pragma unroll
             for (int e = 0; e < 16; ++e) {
                 const int row = m0 + wm * TM + i * 32 + 8 * (e / 4) + c_row_base + (e % 4);
-                if (row < M) C[(size_t)row * N + col] = (half_t)acc[i][j][e];
+                if (row < M) C[(size_t)row * a.ldc + col] = (half_t)acc[i][j][e];
             }
         }
     }
@@ -259,9 +260,10 @@ __global__ void __launch_bounds__(WM* WN * 64) hgemm_f16_dlds_kernel(HgemmArgs a
     // loop would make the compiler treat lgkmcnt as unordered and turn every wait for LDS data into
     // lgkmcnt(0), which also waits for the fragment reads issued just before it.
     float* const partial = a.partial;
+    const int ldc = a.ldc;
     const unsigned rot_tile = (unsigned)a.rot_tile, rot_xcd = (unsigned)a.rot_xcd;
     const int band_m = a.band_m;
-    asm volatile("" ::"s"(partial), "s"(C), "s"(M), "s"(N), "s"(a.kt_per_split), "s"(rot_tile), "s"(rot_xcd), "s"(band_m));
+    asm volatile("" ::"s"(partial), "s"(C), "s"(M), "s"(N), "s"(a.kt_per_split), "s"(rot_tile), "s"(rot_xcd), "s"(band_m), "s"(ldc));
 
     // ---- loader: wavefront-load j of this wavefront covers tile rows (j*NW + wave)*RPW .. +RPW ----
     // A request's address is a wavefront-uniform base (first row of the tile at the K tile wanted, in scalar
@@ -491,7 +493,7 @@ __global__ void __launch_bounds__(WM* WN * 64) hgemm_f16_dlds_kernel(HgemmArgs a
     const int e_col = (lane >> 5) * 4;
     const int row_base = m0 + wm * TM, col_base = n0 + wn * TN;
     constexpr int RS = TN * 2 + 16;          // bytes per staged row of the fp16 epilogue
-    const bool staged = !partial && (N % 8) == 0 && (reinterpret_cast<uintptr_t>(C) & 15u) == 0;
+    const bool staged = !partial && (N % 8) == 0 && (ldc % 8) == 0 && (reinterpret_cast<uintptr_t>(C) & 15u) == 0;
     const int next_vb = vb + (int)gridDim.x;
     const bool has_next_tile = PERSIST && next_vb < total_tiles;
     if (staged || has_next_tile) {
@@ -560,7 +562,7 @@ __global__ void __launch_bounds__(WM* WN * 64) hgemm_f16_dlds_kernel(HgemmArgs a
                 if (lane >= RPR * CH || r >= 32) continue;
                 const half8_t v = *reinterpret_cast<const half8_t*>(region + r * RS + c * 16);
                 const int row = row_base + i * 32 + r, col = col_base + c * 8;
-                if (row < M && col < N) *reinterpret_cast<half8_t*>(C + (size_t)row * N + col) = v;
+                if (row < M && col < N) *reinterpret_cast<half8_t*>(C + (size_t)row * ldc + col) = v;
             }
         }
     } else {
@@ -573,7 +575,7 @@ __global__ void __launch_bounds__(WM* WN * 64) hgemm_f16_dlds_kernel(HgemmArgs a
 #pragma unroll
                 for (int e = 0; e < 16; ++e) {
                     const int col = col_base + j * 32 + (e / 4) * 8 + e_col + (e % 4);
-                    if (col < N) C[(size_t)row * N + col] = (half_t)acc[i][j][e];
+                    if (col < N) C[(size_t)row * ldc + col] = (half_t)acc[i][j][e];
                 }
         }
     }
@@ -702,6 +704,38 @@ static int hgemm_variant_index(const char* name) {
 }
 
 // Measured on MI355X over the Llama2-7B prefill shapes (M in {128, 512, 1024, 2048}), B streamed from HBM.
+// More than 512 rows: the variant with the cheapest schedule and its cost in rounds of 256x256 tiles (see the
+// comment above pick_variant for the constants).
+struct HgemmPlan {
+    int variant;
+    double cost;
+};
+static HgemmPlan plan_many_rows(size_t M, size_t N, size_t K, int cus) {
+    (void)K;
+    static const int v_big = hgemm_variant_index("p256x256x64w2x4s2");
+    static const int v_mid = hgemm_variant_index("p128x256x64w2x4s3");
+    static const int v_small = hgemm_variant_index("p128x128x64w2x4s2");
+    static const int v_few_128x128 = hgemm_variant_index("p128x128x64w2x4s4");
+    static const int v_256x192 = hgemm_variant_index("p256x192x64w2x2s2");
+    auto tiles = [&](int bm, int bn) { return ((M + bm - 1) / bm) * ((N + bn - 1) / bn); };
+    auto cost = [&](size_t t, size_t slots, double round_cost) {
+        const size_t full = t / slots, rem = t % slots;
+        return round_cost * ((double)full + (rem ? 0.65 + 0.3 * (double)rem / (double)slots : 0.0));
+    };
+    const double c_small = cost(tiles(128, 128), (size_t)cus * 2, 0.66);
+    // a problem that leaves half the CUs without a 128x256 tile spreads wider as 128x128 tiles
+    if (tiles(128, 256) * 2 <= (size_t)cus) return {v_few_128x128, c_small};
+    const double c_big = cost(tiles(256, 256), (size_t)cus, 1.0);
+    const double c_mid = cost(tiles(128, 256), (size_t)cus, 0.613);
+    const double c_192 = cost(tiles(256, 192), (size_t)cus, 0.865);   // three quarters of the work at 0.865 of the cost
+    int best = v_big;
+    double c = c_big;
+    if (c_192 < c * 0.97) { best = v_256x192; c = c_192; }
+    if (c_mid < c * 0.97) { best = v_mid; c = c_mid; }
+    if (c_small < c * 0.97) { best = v_small; c = c_small; }
+    return {best, c};
+}
+
 // Up to 512 rows the problem is bound by streaming B once: the largest tile shape that still gives one
 // round of at least 0.6 x CUs workgroups, with a deep (3-4 stage) ring; if even 128x64 tiles are too few,
 // K is split until the chip is full (see launch_hgemm).
@@ -712,15 +746,16 @@ static int hgemm_variant_index(const char* name) {
 // mostly empty; a partly filled round of a fraction f of the CUs costs about (0.65 + 0.3 f) of a full one (fewer
 // busy CUs clock higher).
 // Splitting K or peeling the last round off into a second K-split launch lost to this on every shape tried.
+// What does pay when whole rounds of 256x256 tiles are followed by a mostly empty one: launch the whole rounds as one
+// column range of C and the remaining columns as a second launch with whatever tiles suit THAT problem
+// (launch_hgemm; 2048x11008x4096: 344 big tiles = one round + 88 tiles, or one round + 176 tiles of 128x256).
 static int pick_variant(size_t M, size_t N, size_t K, int cus) {
     static const int v_big = hgemm_variant_index("p256x256x64w2x4s2");
     static const int v_mid = hgemm_variant_index("p128x256x64w2x4s3");
-    static const int v_small = hgemm_variant_index("p128x128x64w2x4s2");
     static const int v_few_256x128 = hgemm_variant_index("p256x128x64w2x4s3");
     static const int v_few_128x128 = hgemm_variant_index("p128x128x64w2x4s4");
     static const int v_few_128x64 = hgemm_variant_index("p128x64x64w4x1s4");
     static const int v_few_128x192 = hgemm_variant_index("p128x192x64w4x2s4");
-    static const int v_256x192 = hgemm_variant_index("p256x192x64w2x2s2");
     auto tiles = [&](int bm, int bn) { return ((M + bm - 1) / bm) * ((N + bn - 1) / bn); };
     if (M <= 512 && tiles(256, 256) <= (size_t)cus) {
         const size_t enough = (size_t)cus * 6 / 10;
@@ -733,26 +768,49 @@ static int pick_variant(size_t M, size_t N, size_t K, int cus) {
         if (tiles(128, 128) >= enough || (K >= 8192 && tiles(128, 128) * 2 >= enough)) return v_few_128x128;
         return v_few_128x64;
     }
-    // a problem that leaves half the CUs without a 128x256 tile spreads wider as 128x128 tiles
-    if (tiles(128, 256) * 2 <= (size_t)cus) return v_few_128x128;
-    auto cost = [&](size_t t, size_t slots, double round_cost) {
-        const size_t full = t / slots, rem = t % slots;
-        return round_cost * ((double)full + (rem ? 0.65 + 0.3 * (double)rem / (double)slots : 0.0));
-    };
-    const double c_big = cost(tiles(256, 256), (size_t)cus, 1.0);
-    const double c_mid = cost(tiles(128, 256), (size_t)cus, 0.613);
-    const double c_small = cost(tiles(128, 128), (size_t)cus * 2, 0.66);
-    const double c_192 = cost(tiles(256, 192), (size_t)cus, 0.865);   // three quarters of the work at 0.865 of the cost
-    int best = v_big;
-    double c = c_big;
-    if (c_192 < c * 0.97) { best = v_256x192; c = c_192; }
-    if (c_mid < c * 0.97) { best = v_mid; c = c_mid; }
-    if (c_small < c * 0.97) { best = v_small; c = c_small; }
-    return best;
+    return plan_many_rows(M, N, K, cus).variant;
 }
+
+// One launch (plus the ordered reduce when K is split) for columns [0, N) of a C whose rows are ldc elements apart.
+// forced_vi: 0 = dispatch by shape.
+static int launch_hgemm_cols(const void* A, const void* B, void* C, size_t M, size_t N, size_t K, size_t ldc, size_t batch,
+                             size_t sa, size_t sb, size_t sc, float** partials_out, int* splits_out,
+                             Workspace::Lease* lease_out, int forced_vi);
 
 int launch_hgemm(const void* A, const void* B, void* C, size_t M, size_t N, size_t K, size_t batch, size_t sa,
                  size_t sb, size_t sc, float** partials_out, int* splits_out, Workspace::Lease* lease_out) {
+    // Whole rounds of 256x256 tiles, then the remaining columns as a problem of their own, when the schedule model
+    // says the two launches beat the best single one.  Only for many rows (no split-K there, so C is written
+    // directly and a column range of it is just a pointer offset with the full row stride).
+    if (batch == 1 && M > 512 && N <= 0x7fffffffu && K > 0 && K % 64 == 0 && K <= ((size_t)1 << 22) && N % 8 == 0 &&
+        aligned16(A) && aligned16(B) && aligned16(C) && g_forced_variant.load() == 0 && g_forced_splits.load() <= 1) {
+        static const int v_big = hgemm_variant_index("p256x256x64w2x4s2");
+        const int cus = device_info().cu_count;
+        const size_t tiles_m = (M + 255) / 256;
+        if (cus > 0 && tiles_m <= (size_t)cus) {
+            const size_t cols_per_round = (size_t)cus / tiles_m, col_tiles = (N + 255) / 256;
+            const size_t full = col_tiles / cols_per_round, rem = col_tiles % cols_per_round;
+            if (full >= 1 && rem > 0) {
+                const size_t N1 = full * cols_per_round * 256;
+                const double whole = plan_many_rows(M, N, K, cus).cost;
+                const double split = (double)full * (double)(tiles_m * cols_per_round) / (double)cus +
+                                     plan_many_rows(M, N - N1, K, cus).cost + 0.04;   // 0.04: the second launch's ramp
+                if (split < whole * 0.97) {
+                    int rc = launch_hgemm_cols(A, B, C, M, N1, K, N, 1, 0, 0, 0, nullptr, nullptr, nullptr, v_big);
+                    if (rc != TL_OK) return rc;
+                    if (splits_out) *splits_out = 1;
+                    return launch_hgemm_cols(A, (const half_t*)B + N1 * K, (half_t*)C + N1, M, N - N1, K, N, 1, 0, 0, 0,
+                                             nullptr, nullptr, nullptr, 0);
+                }
+            }
+        }
+    }
+    return launch_hgemm_cols(A, B, C, M, N, K, N, batch, sa, sb, sc, partials_out, splits_out, lease_out, 0);
+}
+
+static int launch_hgemm_cols(const void* A, const void* B, void* C, size_t M, size_t N, size_t K, size_t ldc, size_t batch,
+                             size_t sa, size_t sb, size_t sc, float** partials_out, int* splits_out,
+                             Workspace::Lease* lease_out, int forced_vi) {
     Workspace::Lease own_lease;
     Workspace::Lease& lease = lease_out ? *lease_out : own_lease;
     if (splits_out) *splits_out = 1;
@@ -770,6 +828,7 @@ int launch_hgemm(const void* A, const void* B, void* C, size_t M, size_t N, size
     const bool vec_ok = (K % 8 == 0) && aligned16(A) && aligned16(B) &&
                         (batch == 1 || (sa % 8 == 0 && sb % 8 == 0));
     if (!vec_ok) {
+        TL_REQUIRE(ldc == N, "hgemm generic path: a column range of C is not supported");
         dim3 grid((unsigned)((N + 15) / 16), (unsigned)((M + 15) / 16), (unsigned)batch);
         TL_REQUIRE(grid.y <= 65535, "hgemm generic path: M too large (%zu)", M);
         hipLaunchKernelGGL((gemm_generic_kernel<half_t, float>), grid, dim3(256), 0, st, (const half_t*)A,
@@ -777,7 +836,7 @@ int launch_hgemm(const void* A, const void* B, void* C, size_t M, size_t N, size
         TL_CHECK_LAUNCH("gemm_generic_kernel<half>");
         return TL_OK;
     }
-    const int forced_variant = g_forced_variant.load();
+    const int forced_variant = forced_vi ? forced_vi : g_forced_variant.load();
     int vi = forced_variant ? forced_variant : pick_variant(M, N, K, device_info().cu_count);
     if (g_variants[vi].stages > 0 && K % g_variants[vi].bk != 0) vi = 1;  // direct-to-LDS path cannot zero-fill a K tail
     // its per-lane byte offsets inside a tile ((rows - 1) * K + 64 halves) are 32-bit
@@ -795,6 +854,7 @@ int launch_hgemm(const void* A, const void* B, void* C, size_t M, size_t N, size
     a.C = (half_t*)C;
     a.M = (int)M;
     a.N = (int)N;
+    a.ldc = (int)ldc;
     a.K = (int)K;
     a.tiles_m = (int)((M + v.bm - 1) / v.bm);
     a.tiles_n = (int)((N + v.bn - 1) / v.bn);
@@ -828,7 +888,7 @@ int launch_hgemm(const void* A, const void* B, void* C, size_t M, size_t N, size
             if (splits < 1) splits = 1;
         }
         if (splits > KT) splits = KT;
-        if (batch != 1) splits = 1;
+        if (batch != 1 || ldc != N) splits = 1;   // the reduce pass writes a dense C
         if (splits > 1) {
             a.kt_per_split = (KT + splits - 1) / splits;
             splits = (KT + a.kt_per_split - 1) / a.kt_per_split;

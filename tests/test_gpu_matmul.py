@@ -166,6 +166,26 @@ def test_hgemm_prefill_whole_matrix_against_second_gpu_path(dev, oracle, M, N, K
     assert float((err > 0).float().mean()) < 0.2, "an unexpected share of entries rounds differently"
 
 
+@pytest.mark.parametrize("M,N,K", [(2048, 8328, 128), (1100, 16520, 64), (2048, 8192 + 8, 192)])
+def test_hgemm_column_range_split_launches(dev, oracle, M, N, K):
+    """Shapes whose 256x256 tiles fill whole rounds of the chip plus a nearly empty one are issued as two launches
+    over two column ranges of C (row stride N in both): every entry is written, matches the plain fp32 kernel inside
+    the parity gate, and whole rows (which cross the seam) match the oracle."""
+    A = synth.normal_f16(2100 + M, (M, K), 1.0)
+    B = synth.normal_f16(2101 + N % 89, (N, K), 0.05)
+    Ad, Bd = dev.from_numpy(A), dev.from_numpy(B)
+    ref = dev.matmul2d_f32(Ad.float(), Bd.float()).half()
+    C = dev.empty(M, N)
+    C.fill_(float("nan"))
+    dev.hgemm(Ad, Bd, C)
+    assert not bool(torch.isnan(C).any()), "entries left unwritten"
+    rows = np.array([0, 255, 256, M - 1])
+    assert_close_f16(C.cpu().numpy()[rows], oracle.matmul2d(A[rows], B), RTOL, ATOL, "rows against the oracle")
+    err = (C.float() - ref.float()).abs()
+    assert bool((err <= ATOL + RTOL * ref.float().abs()).all())
+    assert float((err > 0).float().mean()) < 0.2
+
+
 def test_hgemm_every_variant_ragged(dev, oracle):
     names = dev.hgemm_variants()
     for v in range(1, len(names)):
