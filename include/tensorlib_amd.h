@@ -121,6 +121,10 @@ int tl_set_hgemm_tile_band(int band);
 /* Tuning hook: prefill attention kernel, 0 = automatic, 1 = one wavefront per 32 query rows,
  * 2 = LDS-tiled workgroups of 128 query rows (head_dim 128, ldv covering the context rounded up to 64). */
 int tl_set_prefill_attention_variant(int variant);
+/* Tuning hook: where the chunk partials of the decode attention are merged: 0 = automatic (inside the one launch
+ * up to 512 cached positions), 1 = always inside the launch, by the workgroup that finishes a head's last chunk,
+ * 2 = always by a second launch.  Same bits either way. */
+int tl_set_decode_attention_merge(int mode);
 /* Tuning hook: cap the GEMV grid at `waves` resident wavefronts per compute unit (0 = default). */
 int tl_set_gemv_grid_waves_per_cu(int waves);
 

@@ -20,6 +20,13 @@ namespace tl {
 
 // 0: automatic, 1: one wavefront per 32 query rows, 2: LDS-tiled workgroups of 128 query rows (tuning hook)
 static std::atomic<int> g_prefill_attention_variant{0};
+// where the chunk partials of a head are merged: 0 = automatic, 1 = by the workgroup that finishes the head's last
+// chunk, 2 = by a second launch
+static std::atomic<int> g_decode_merge_mode{0};
+// Up to this many chunks the in-kernel merge is ahead (384 positions: 7.6 against 10.2 us for the pair of launches;
+// 1024 positions: equal; 1951 positions: 14.7 against 13.2 us, the merging workgroup's serial walk over 31 partials
+// through device-coherent loads then costs more than a launch).
+constexpr int kMergeInKernelMaxChunks = 8;
 
 template <int CTRL>
 __device__ __forceinline__ float dppf(float v) {
@@ -81,6 +88,48 @@ __global__ void __launch_bounds__(256) rope_table_kernel(half_t* table, int max_
     *reinterpret_cast<half2_t*>(table + 2 * i) = cs;
 }
 
+// Merge of the chunk partials of head h for output dimension d (base: the head's first partial).  COHERENT: the
+// partials were written by other workgroups of the SAME launch and are read with device-coherent loads.
+template <bool COHERENT>
+__device__ __forceinline__ void merge_head(half_t* out, const float* base, int h, int D, int n_chunks, int d) {
+    auto ldp = [](const float* p) {
+        if constexpr (COHERENT) return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        else return *p;
+    };
+    // Sixteen chunks per round trip (a long context has dozens of chunks, and a dependent load per chunk would
+    // cost a memory latency each), folded in with the online-softmax update, so the maxima need no pass of their
+    // own; the sums run over the chunks in ascending order.
+    constexpr int U = 16;
+    float m = -INFINITY, l = 0.f, o = 0.f;
+    for (int c0 = 0; c0 < n_chunks; c0 += U) {
+        float pm[U], pl[U], po[U];
+#pragma unroll
+        for (int j = 0; j < U; ++j) {
+            const float* p = base + (size_t)(c0 + j < n_chunks ? c0 + j : c0) * (D + 2);
+            pm[j] = ldp(p);
+            pl[j] = ldp(p + 1);
+            po[j] = ldp(p + 2 + d);
+        }
+        float m_new = m;
+#pragma unroll
+        for (int j = 0; j < U; ++j)
+            if (c0 + j < n_chunks) m_new = fmaxf(m_new, pm[j]);
+        const float scale = expf(m - m_new);   // 0 on the first round (m = -inf), 1 when the maximum stays
+        l *= scale;
+        o *= scale;
+        m = m_new;
+#pragma unroll
+        for (int j = 0; j < U; ++j) {
+            if (c0 + j < n_chunks) {
+                const float w = expf(pm[j] - m);
+                l = __builtin_fmaf(pl[j], w, l);
+                o = __builtin_fmaf(po[j], w, o);
+            }
+        }
+    }
+    out[(size_t)h * D + d] = (half_t)(o / l);
+}
+
 // FUSE_ROPE: `q` points at the raw q|k|v projection of the new token (position T-1).  q is rotated
 // on load; the workgroup that owns the last chunk rotates the new k row, uses it, and writes it and
 // the new v row into the caches (each head's workgroup writes only its own head slice).
@@ -90,7 +139,7 @@ template <int LPR, int ROPE>
 __global__ void __launch_bounds__(kAttnThreads)
 decode_attn_partial_kernel(half_t* out, float* partial, const half_t* q, half_t* cache_k,
                            half_t* cache_v, const half_t* rope_table, int T, int n_heads, float inv_scale,
-                           int n_chunks) {
+                           int n_chunks, unsigned* tickets) {
     constexpr int D = LPR * 8;
     constexpr int GROUPS = kAttnThreads / LPR;
     __shared__ float sc[kAttnChunk];
@@ -212,55 +261,48 @@ decode_attn_partial_kernel(half_t* out, float* partial, const half_t* q, half_t*
             out[(size_t)h * D + tid] = (half_t)(o / l);
         } else {
             float* p = partial + ((size_t)h * n_chunks + chunk) * (D + 2);
-            p[2 + tid] = o;
-            if (tid == 0) { p[0] = m; p[1] = l; }
+            if (tickets) {
+                // device-coherent stores: the workgroup that merges may sit on another XCD, behind another L2
+                __hip_atomic_store(p + 2 + tid, o, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                if (tid == 0) {
+                    __hip_atomic_store(p, m, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    __hip_atomic_store(p + 1, l, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                }
+            } else {
+                p[2 + tid] = o;
+                if (tid == 0) { p[0] = m; p[1] = l; }
+            }
         }
     }
+    if (tickets == nullptr || n_chunks == 1) return;
+    // One launch instead of two: the workgroup that finishes a head's last chunk merges the head.  Its partials
+    // have been acknowledged (vmcnt(0)) before its ticket is drawn, tickets and partials are device-coherent
+    // accesses, and the merge walks the chunks in index order, so the result has the bits of the two-launch path.
+    __shared__ int s_last;
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    if (tid == 0) {
+        const unsigned t = __hip_atomic_fetch_add(tickets + h, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        const int last = (t + 1u == (unsigned)n_chunks);
+        if (last) __hip_atomic_store(tickets + h, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // ready for the next call
+        s_last = last;
+    }
+    __syncthreads();
+    if (!s_last || tid >= D) return;
+    merge_head<true>(out, partial + (size_t)h * n_chunks * (D + 2), h, D, n_chunks, tid);
 }
 
-// Second pass: merge the chunk partials of one head.  (Folding this into the first launch with a
-// "last workgroup merges" ticket was measured slower: the device-scope fences it needs cost more
-// than this 4 us launch.  So was one 1024-thread workgroup per head covering up to 512 positions
-// alone: 32 workgroups pull a context through 32 CUs' L2 ports instead of 256, and a whole decode
-// step lost 6 %.)
+// Second pass for long contexts: merge the chunk partials of one head.  (Short contexts merge inside the first
+// launch, see the ticket at the end of decode_attn_partial_kernel.  Doing that with device-scope fences around
+// plain accesses instead of device-coherent accesses cost 18 us against 12.6 us for two launches: the fences write
+// back and invalidate whole L2s.  One 1024-thread workgroup per head covering up to 512 positions alone was slower
+// too: 32 workgroups pull a context through 32 CUs' L2 ports instead of 256, and a whole decode step lost 6 %.)
 __global__ void __launch_bounds__(256)
 decode_attn_merge_kernel(half_t* out, const float* partial, int D, int n_chunks) {
     const int h = blockIdx.x;
     const int d = threadIdx.x;
     if (d >= D) return;
-    const float* base = partial + (size_t)h * n_chunks * (D + 2);
-    // Sixteen chunks per round trip (a long context has dozens of chunks, and a dependent load per chunk would
-    // cost a memory latency each), folded in with the online-softmax update, so the maxima need no pass of their
-    // own; the sums run over the chunks in ascending order.
-    constexpr int U = 16;
-    float m = -INFINITY, l = 0.f, o = 0.f;
-    for (int c0 = 0; c0 < n_chunks; c0 += U) {
-        float pm[U], pl[U], po[U];
-#pragma unroll
-        for (int j = 0; j < U; ++j) {
-            const float* p = base + (size_t)(c0 + j < n_chunks ? c0 + j : c0) * (D + 2);
-            pm[j] = p[0];
-            pl[j] = p[1];
-            po[j] = p[2 + d];
-        }
-        float m_new = m;
-#pragma unroll
-        for (int j = 0; j < U; ++j)
-            if (c0 + j < n_chunks) m_new = fmaxf(m_new, pm[j]);
-        const float scale = expf(m - m_new);   // 0 on the first round (m = -inf), 1 when the maximum stays
-        l *= scale;
-        o *= scale;
-        m = m_new;
-#pragma unroll
-        for (int j = 0; j < U; ++j) {
-            if (c0 + j < n_chunks) {
-                const float w = expf(pm[j] - m);
-                l = __builtin_fmaf(pl[j], w, l);
-                o = __builtin_fmaf(po[j], w, o);
-            }
-        }
-    }
-    out[(size_t)h * D + d] = (half_t)(o / l);
+    merge_head<false>(out, partial + (size_t)h * n_chunks * (D + 2), h, D, n_chunks, d);
 }
 
 // mask[r, i, j] = (j > start_pos + i) ? -inf : 0 for r < reps, i < seqlen, j < start_pos + seqlen
@@ -887,11 +929,13 @@ static int launch_decode_attention(void* out, const void* q, void* cache_k, void
     const int n_chunks = (T + tl::kAttnChunk - 1) / tl::kAttnChunk;
     TL_REQUIRE(n_chunks <= 65535, "%s: T=%d too long", name, T);
     tl::Workspace::Lease lease;   // held until both kernels are enqueued
-    const size_t ws_floats = (size_t)n_heads * n_chunks * (head_dim + 2);
+    // [one ticket per head, padded to 64 words][partials]; tickets are zero between calls
+    const size_t ticket_words = ((size_t)n_heads + 63) / 64 * 64;
+    const size_t ws_floats = ticket_words + (size_t)n_heads * n_chunks * (head_dim + 2);
     float* ws = static_ws;
     if (static_ws) {
         TL_REQUIRE(ws_floats <= static_ws_floats,
-                   "%s: %d heads x %d chunks of 64 positions x (%d + 2) floats = %zu floats of partial results exceed the "
+                   "%s: %d heads x %d chunks of 64 positions x (%d + 2) floats (+ tickets) = %zu floats of partial results exceed the "
                    "static scratch of %zu floats; use tl_decode_attention_rope_f16 for this size",
                    name, n_heads, n_chunks, head_dim, ws_floats, static_ws_floats);
     } else if (n_chunks > 1) {
@@ -899,15 +943,19 @@ static int launch_decode_attention(void* out, const void* q, void* cache_k, void
         if (rc != TL_OK) return rc;
         ws = lease.ptr;
     }
+    const int merge_mode = tl::g_decode_merge_mode.load();
+    const bool in_kernel = merge_mode == 1 || (merge_mode == 0 && n_chunks <= tl::kMergeInKernelMaxChunks);
+    unsigned* tickets = (ws && in_kernel) ? reinterpret_cast<unsigned*>(ws) : nullptr;
+    float* partials = ws ? ws + ticket_words : nullptr;
     // the reference divides the scores by half(sqrt(head_dim)) (Transformer.cpp:94)
     const float scale = (float)(tl::half_t)sqrtf((float)head_dim);
     const float inv_scale = 1.0f / scale;
     dim3 grid(n_heads, n_chunks);
     hipStream_t st = tl::stream();
     auto launch = [&](auto kernel) {
-        hipLaunchKernelGGL(kernel, grid, dim3(tl::kAttnThreads), 0, st, (tl::half_t*)out, ws,
+        hipLaunchKernelGGL(kernel, grid, dim3(tl::kAttnThreads), 0, st, (tl::half_t*)out, partials,
                            (const tl::half_t*)q, (tl::half_t*)cache_k, (tl::half_t*)cache_v,
-                           (const tl::half_t*)rope_table, T, n_heads, inv_scale, n_chunks);
+                           (const tl::half_t*)rope_table, T, n_heads, inv_scale, n_chunks, tickets);
     };
     if (fuse_rope && rope_table) {
         if (head_dim == 64) launch(tl::decode_attn_partial_kernel<8, 1>);
@@ -923,8 +971,8 @@ static int launch_decode_attention(void* out, const void* q, void* cache_k, void
         else launch(tl::decode_attn_partial_kernel<32, 0>);
     }
     TL_CHECK_LAUNCH("decode_attn_partial_kernel");
-    if (n_chunks > 1) {
-        hipLaunchKernelGGL(tl::decode_attn_merge_kernel, dim3(n_heads), dim3(256), 0, st, (tl::half_t*)out, ws, head_dim,
+    if (n_chunks > 1 && !tickets) {
+        hipLaunchKernelGGL(tl::decode_attn_merge_kernel, dim3(n_heads), dim3(256), 0, st, (tl::half_t*)out, partials, head_dim,
                            n_chunks);
         TL_CHECK_LAUNCH("decode_attn_merge_kernel");
     }
@@ -1078,6 +1126,12 @@ int tl_prefill_attention_f16(void* out, const void* q, const void* cache_k, cons
                            (const tl::half_t*)q, (const tl::half_t*)cache_k, (const tl::half_t*)vT, ldv, start_pos, n_tokens,
                            n_heads, divisor);
     TL_CHECK_LAUNCH("prefill_attention_kernel");
+    return TL_OK;
+}
+
+int tl_set_decode_attention_merge(int mode) {
+    TL_REQUIRE(mode >= 0 && mode <= 2, "tl_set_decode_attention_merge: %d out of range [0,2]", mode);
+    tl::g_decode_merge_mode = mode;
     return TL_OK;
 }
 

@@ -82,6 +82,8 @@ int Workspace::acquire(size_t floats, size_t min_floats, const char* what, Lease
                              hipGetErrorString(e));
         }
         floats_ = want;
+        // users keep counters in the buffer that are zero between calls (attention tickets): start from zeros
+        TL_HIP_TRY(hipMemsetAsync(ptr_, 0, want * sizeof(float), st));
     }
     last_stream_ = st;
     used_ = true;

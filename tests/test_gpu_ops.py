@@ -358,6 +358,27 @@ def test_rope_table_bits_equal_the_cpu_loop(dev, oracle, D):
     assert differs.shape == (2048, D // 2) and not differs[0].any()
 
 
+@pytest.mark.parametrize("T", [65, 200, 512, 513, 1500])
+def test_decode_attention_merge_inside_the_launch_equals_second_launch(dev, T):
+    """The chunk partials of a head are merged either by the workgroup that finishes the head's last chunk (tickets,
+    device-coherent partials) or by a second launch: same chunk order, so the same bits; repeated calls show that
+    the tickets return to zero."""
+    H, D = 32, 128
+    q = dev.from_numpy(synth.normal_f16(150, (H, D), 1.0))
+    ck = dev.from_numpy(synth.normal_f16(151, (T, H, D), 1.0))
+    cv = dev.from_numpy(synth.normal_f16(152, (T, H, D), 1.0))
+    try:
+        dev.lib.tl_set_decode_attention_merge(2)
+        want = dev.decode_attention(q, ck, cv, T)
+        dev.lib.tl_set_decode_attention_merge(1)
+        for _ in range(3):
+            assert torch.equal(dev.decode_attention(q, ck, cv, T), want)
+        dev.lib.tl_set_decode_attention_merge(0)
+        assert torch.equal(dev.decode_attention(q, ck, cv, T), want)
+    finally:
+        dev.lib.tl_set_decode_attention_merge(0)
+
+
 def test_decode_attention_repeated_calls_reuse_counters(dev, oracle):
     """Many calls in a row with different numbers of chunks share one partials workspace: all of
     them have to agree with the CPU chain."""
