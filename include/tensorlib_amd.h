@@ -228,10 +228,12 @@ int tl_decode_attention_rope_f16(void* out, const void* qkv, void* cache_k, void
  * results; the per-chunk partial results go to a static device array of TL_DECODE_ATTENTION_STATIC_SCRATCH_FLOATS
  * floats that is part of the library's code object (each GPU holds its copy until the process ends) instead of the
  * grown-on-demand workspace, and the call makes no hipMalloc / hipFree.  Limit:
- *   n_heads * ceil((pos + 1) / 64) * (head_dim + 2) <= TL_DECODE_ATTENTION_STATIC_SCRATCH_FLOATS
+ *   64 * ceil(n_heads / 64) + n_heads * ceil((pos + 1) / 64) * (head_dim + 2) <= TL_DECODE_ATTENTION_STATIC_SCRATCH_FLOATS
  * (32 heads of 128: 16128 positions); larger sizes return TL_EINVAL.  Every call on a GPU shares that GPU's array:
- * calls that overlap on one GPU (two streams, two host threads) race; calls on one stream do not.  Nothing in the
- * array has to start at zero (every slot a call reads was written by the same call). */
+ * calls that overlap on one GPU (two streams, two host threads) race; calls on one stream do not.  The caller clears
+ * nothing: every partial a call reads was written by the same call, and the per-head tickets at the head of the array
+ * (64 words per 64 heads, counted in the limit) are zero when the library is loaded and are set back to zero by the
+ * workgroup that draws a head's last one. */
 #define TL_DECODE_ATTENTION_STATIC_SCRATCH_FLOATS (1u << 20)
 int tl_decode_attention_rope_static_f16(void* out, const void* qkv, void* cache_k, void* cache_v,
                                         const void* rope_table, int pos, int n_heads, int head_dim);
