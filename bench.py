@@ -16,7 +16,8 @@ against the MFMA rate this chip sustains out of registers) and Llama2-7B decode 
 
 `--workload hgemm` times only the prefill HGEMM shapes (step = one pass over the M=2048 shapes)
 and prints the same kind of line with an MFMA roofline; it exists so that the MFMA profile under
-profiles/ can be taken from a committed command.
+profiles/ can be taken from a committed command.  `--workload decode` does the same for the
+Llama2-7B decode step (step = one generated token of the fused driver after a 128-token prompt).
 """
 from __future__ import annotations
 
@@ -53,7 +54,7 @@ def parse_args():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", choices=["gemv", "hgemm"], default="gemv")
+    ap.add_argument("--workload", choices=["gemv", "hgemm", "decode"], default="gemv")
     ap.add_argument("--no-extra", action="store_true", help="skip the HGEMM / per-shape / model extras")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--copy-calibration", action="store_true",
@@ -235,6 +236,33 @@ def main():
 
     def randn(shape, std):
         return (torch.randn(shape, generator=gen, device="cuda", dtype=torch.float32) * std).to(torch.float16)
+
+    if args.workload == "decode":
+        from tensorlib_amd import llama2
+        cfg = llama2.Llama2Config()
+        m = llama2.Llama2Model(dev, cfg, max_tokens=128)
+        m.random_init_on_device(seed=7)
+        prompt = synth.token_ids(11, 128, cfg.vocab_size)
+        m.generate(prompt, max(2, args.warmup), llama2.MODE_FUSED)
+        _, tp, td = m.generate(prompt, args.steps + 1, llama2.MODE_FUSED)   # the first token comes out of the prefill
+        tok_s = args.steps / td
+        wbytes = cfg.weight_bytes_per_token()
+        out = {
+            "metric": "Llama2-7B decode tok/s (fused driver, batch 1)", "value": round(tok_s, 2), "unit": "tok/s",
+            "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(1e3 / tok_s, 5),
+            "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16", "data": "synthetic",
+            "config": {"workload": f"Llama2-7B fp16 random-init, 128-token random prompt, {args.steps} greedy decode steps, "
+                                   "batch 1, max_seq 2048", "weight_bytes_per_token": wbytes},
+            "roofline": {"bound": "hbm", "achieved": round(wbytes * tok_s / 1e9, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                         "frac": round(wbytes * tok_s / 1e9 / HBM_PEAK_GBS, 4), "traffic": None,
+                         "kernel": "whole decode step (weight bytes per token x tok/s)"},
+            "extra": {"prefill_tok_s": round(128 / tp, 1)},
+        }
+        m.close()
+        if not args.no_cpu:
+            out["cpu_baseline"] = cpu_baseline_llama2_decode()
+        print(json.dumps(out))
+        return
 
     if args.workload == "hgemm":
         shapes = [s for s in HGEMM_SHAPES if s[0] == 2048]
