@@ -268,7 +268,7 @@ class Llama2Model:
 
 
 def bench_decode(dev, n_prompt: int = 128, n_generate: int = 256) -> dict:
-    """BASELINE config 4: full Llama2-7B, random-init fp16 weights, 128-token random prompt,
+    """Full Llama2-7B, random-init fp16 weights, 128-token random prompt,
     256 greedy steps, batch 1, max_seq 2048."""
     from . import synth
     cfg = Llama2Config()

@@ -167,7 +167,7 @@ def test_driver_rejects_bad_calls(dev):
 
 
 def test_llama2_7b_block_decode_kv1024_and_prefill_512(dev):
-    """BASELINE config 3: one transformer block at Llama2-7B size."""
+    """One transformer block at Llama2-7B size."""
     from tensorlib_amd.llama2 import (BUF_CACHE_K, BUF_CACHE_V, BUF_X, MODE_FUSED, MODE_REFERENCE_CHAIN, Llama2Config,
                                       Llama2Model)
     cfg = Llama2Config(dim=4096, hidden_dim=11008, n_layers=1, n_heads=32, vocab_size=512, max_seq_len=2048)
@@ -209,7 +209,7 @@ def test_llama2_7b_block_decode_kv1024_and_prefill_512(dev):
 
 
 def test_llama2_7b_full_model(dev):
-    """BASELINE config 4: 32 layers, vocab 32000, random-init fp16 weights.  Logits parity on a
+    """32 layers, vocab 32000, random-init fp16 weights.  Logits parity on a
     short teacher-forced sequence (the O(MNK) CPU oracle needs ~7 G multiply-adds per token),
     then the full 128-token prefill + 256 greedy steps in both modes with size-independent checks."""
     from tensorlib_amd.llama2 import MODE_FUSED, MODE_REFERENCE_CHAIN, Llama2Config, Llama2Model

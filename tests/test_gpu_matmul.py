@@ -36,13 +36,13 @@ def _gemv_case(dev, oracle, N, K, seed, variant=0, w_std=0.02):
 
 
 def test_gemv_config_single(dev, oracle):
-    """BASELINE config 0: W[4096,4096] ~ N(0,0.02), x ~ N(0,1)."""
+    """W[4096,4096] ~ N(0,0.02), x ~ N(0,1)."""
     _gemv_case(dev, oracle, 4096, 4096, seed=100)
 
 
 @pytest.mark.parametrize("N,K", SWEEP)
 def test_gemv_decode_sweep(dev, oracle, N, K):
-    """BASELINE config 1: the four Llama2-7B decode shapes, through matmul2d with M == 1."""
+    """The four Llama2-7B decode shapes, through matmul2d with M == 1."""
     W = synth.normal_f16(200 + N % 97, (N, K), 0.02)
     x = synth.normal_f16(300 + K % 89, (1, K), 1.0)
     y = dev.matmul2d(dev.from_numpy(x), dev.from_numpy(W)).cpu().numpy()
@@ -131,7 +131,7 @@ def test_hgemm_prefill_full_oracle(dev, oracle, M, N, K):
 @pytest.mark.parametrize("M", [128, 512, 2048])
 @pytest.mark.parametrize("N,K", [(4096, 4096), (11008, 4096), (32000, 4096), (4096, 11008)])
 def test_hgemm_prefill_shapes_sampled(dev, oracle, M, N, K):
-    """BASELINE config 2 at full size: oracle on sampled rows and entries."""
+    """The twelve prefill shapes at full size: oracle on sampled rows and entries."""
     _hgemm_case(dev, oracle, M, N, K, seed=900 + M + N % 31, full=False)
 
 
