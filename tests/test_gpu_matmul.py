@@ -369,3 +369,48 @@ def test_linearity_at_full_size(dev):
     y2 = dev.gemv(dev.from_numpy(x2), Wd).float()
     y12 = dev.gemv(dev.from_numpy((x1 + x2).astype(np.float16)), Wd).float()
     assert torch.equal(y12, y1 + y2)
+
+
+def test_split_k_workspace_shared_by_two_host_threads(dev):
+    """Two host threads issue split-K GEMMs of growing size at the same time (the reference's Embedding::forward
+    enters the backend from an OpenMP loop, tensorLib/src/nn/embedding.cpp:66-78).  Both use the one library-owned
+    fp32 workspace, which has to grow several times meanwhile: a call keeps the buffer locked until its kernels are
+    enqueued, so no thread can free it under another thread's queued kernel.  Every result is compared with the
+    single-threaded one."""
+    import threading
+    K = 4096
+    sizes = [(128, 1024), (96, 4096), (128, 8192), (128, 16384), (70, 2048), (128, 24576)]
+    jobs = []
+    dev.lib.tl_set_hgemm_splits(4)
+    try:
+        for i, (M, N) in enumerate(sizes):
+            A = dev.from_numpy(synth.normal_f16(2300 + i, (M, K), 1.0))
+            B = dev.from_numpy(synth.normal_f16(2400 + i, (N, K), 0.02))
+            jobs.append((A, B, dev.hgemm(A, B).clone()))
+    finally:
+        dev.lib.tl_set_hgemm_splits(0)
+    dev.synchronize()
+    errors = []
+
+    def worker(order):
+        try:
+            for _ in range(3):
+                for j in order:
+                    A, B, want = jobs[j]
+                    C = dev.hgemm(A, B)
+                    dev.synchronize()
+                    if not torch.equal(C, want):
+                        errors.append(f"job {j} differs")
+        except Exception as e:   # noqa: BLE001
+            errors.append(repr(e))
+
+    dev.lib.tl_set_hgemm_splits(4)
+    try:
+        ts = [threading.Thread(target=worker, args=(o,)) for o in ([0, 1, 2, 3, 4, 5], [5, 3, 1, 4, 2, 0])]
+        for t in ts:
+            t.start()
+        for t in ts:
+            t.join()
+    finally:
+        dev.lib.tl_set_hgemm_splits(0)
+    assert not errors, errors[:3]
