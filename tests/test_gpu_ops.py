@@ -534,3 +534,31 @@ def test_prefill_attention_limits(dev):
     from tensorlib_amd import TensorLibError
     with pytest.raises(TensorLibError):
         dev.prefill_attention(dev.empty(2, 4, 256), dev.empty(8, 2, 256), dev.empty(8, 2, 256), 0)   # head_dim 256
+
+
+def test_empty_inputs_are_accepted_and_touch_nothing(dev):
+    """Zero rows / tokens / elements through the C ABI: every op returns success without a launch (the reference's
+    Tensor layer can hand over empty views, e.g. a zero-length slice), and a canary buffer keeps its bits."""
+    import ctypes
+    from tensorlib_amd._lib import check
+    lib = dev.lib
+    canary = dev.from_numpy(synth.normal_f16(990, (64,), 1.0))
+    before = canary.clone()
+    p = ctypes.c_void_p(canary.data_ptr())
+    ids = torch.zeros(4, dtype=torch.int32, device=canary.device)
+    ip = ctypes.c_void_p(ids.data_ptr())
+    check(lib.tl_rms_norm_f16(p, p, p, 1e-5, 64, 0), "rms_norm, no tokens")
+    check(lib.tl_apply_rotary_emb_f16(p, p, 0, 1, 0, 2, 32), "rope, no positions")
+    check(lib.tl_softmax_f16(p, p, 0, 64), "softmax, no rows")
+    check(lib.tl_softmax_f16(p, p, 4, 0), "softmax, no columns")
+    check(lib.tl_silu_f16(p, p, 0), "silu, no elements")
+    check(lib.tl_silu_mul_f16(p, p, p, 0), "silu_mul, no elements")
+    check(lib.tl_binary_f16(p, p, p, 0, 0), "binary, no elements")
+    check(lib.tl_binary_scalar_f16(p, p, 0x3c00, 0, 3), "binary scalar, no elements")
+    check(lib.tl_full_f16(p, 0x3c00, 0), "full, no elements")
+    check(lib.tl_embedding_f16(p, p, ip, 0, 16, 4), "embedding, no tokens")
+    check(lib.tl_gemv_f16(p, p, p, 0, 64), "gemv, no rows")
+    check(lib.tl_causal_mask_f16(p, 0, 4, 0), "mask, no repetitions")
+    check(lib.tl_add_rms_norm_f16(p, p, p, p, p, 1e-5, 64, 0), "add_rms_norm, no tokens")
+    dev.synchronize()
+    assert torch.equal(canary, before)
