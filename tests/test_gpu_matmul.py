@@ -220,6 +220,29 @@ def test_hgemm_integer_inputs_bit_exact(dev, oracle):
     assert np.array_equal(C.astype(np.float64), ref)
 
 
+def test_matmul2d_drawn_shapes_integer_exact(dev):
+    """Sixty shapes drawn with a fixed seed from the edges of every dispatch rule (M = 1 and few rows, N and K around
+    the tile sizes, multiples of 8 and 64 and odd values) through the boundary entry; small-integer inputs make every
+    sum exact in fp32 and in fp16, so a wrong index, a skipped tail or a stale tile shows as a wrong value.  The
+    expected values come from float64 on the host."""
+    import random
+    rnd = random.Random(20240611)
+    Ms = [1, 2, 3, 15, 16, 17, 31, 33, 64, 100, 128, 129, 255, 256, 300, 512, lambda: rnd.randint(1, 700)]
+    Ns = [1, 7, 8, 16, 48, 63, 64, 65, 128, 200, 256, 320, 1000, 1024, lambda: rnd.randint(1, 3000), lambda: 8 * rnd.randint(1, 400)]
+    Ks = [1, 7, 8, 24, 64, 72, 128, 192, 256, 320, 512, 1000, 1024, lambda: rnd.randint(1, 3000), lambda: 8 * rnd.randint(1, 300),
+          lambda: 64 * rnd.randint(1, 60)]
+    pick = lambda xs: (lambda c: c() if callable(c) else c)(rnd.choice(xs))
+    for i in range(60):
+        M, N, K = pick(Ms), pick(Ns), pick(Ks)
+        A = synth.small_ints_f16(7000 + 2 * i, (M, K), -2, 2)
+        B = synth.small_ints_f16(7001 + 2 * i, (N, K), -2, 2)
+        C = torch.full((M, N), 5.0, device="cuda", dtype=torch.float16)
+        dev.matmul2d(dev.from_numpy(A), dev.from_numpy(B), C)
+        want = A.astype(np.float64) @ B.astype(np.float64).T
+        assert np.abs(want).max() <= 2048, (M, N, K)           # every sum is an fp16 integer
+        assert np.array_equal(C.cpu().numpy().astype(np.float64), want), (i, M, N, K)
+
+
 def test_hgemm_k_rotation_and_splits_visit_every_k_tile_once(dev, oracle):
     """Workgroups start their walk over K at a rotated tile and wrap, per split: with small-integer data the
     result is exact whatever the order, so a skipped or repeated K tile shows as a wrong bit."""
