@@ -186,9 +186,9 @@ def mfma_sustained(dev):
     return out
 
 
-def hgemm_table(dev, randn, torch, synth, sustained_tf):
+def hgemm_table(dev, randn, torch, synth, sustained_tf, shapes=None):
     hg = {}
-    for (M, N, K) in HGEMM_SHAPES:
+    for (M, N, K) in (shapes or HGEMM_SHAPES):
         A = randn((M, K), 1.0)
         # W rotates over enough copies (>= 600 MB) that every launch streams it from HBM, as a forward pass
         # over 32 layers does; one 33-180 MB matrix used again and again would sit in the 256 MB memory-side cache
@@ -408,6 +408,9 @@ def main():
         sustained = mfma_sustained(dev)
         extra["mfma_sustained_tflops"] = sustained
         extra["hgemm_prefill"] = hgemm_table(dev, randn, torch, synth, sustained["changing_operands"])
+        # a prompt of a few tokens (the reference's usual prefill): the projections of a 16-token prompt
+        extra["hgemm_short_prompt"] = hgemm_table(dev, randn, torch, synth, sustained["changing_operands"],
+                                                  [(16, 12288, 4096), (16, 4096, 4096), (16, 22016, 4096), (16, 4096, 11008)])
         torch.cuda.empty_cache()
         from tensorlib_amd import llama2
         extra["llama2_7b_decode"] = llama2.bench_decode(dev)

@@ -118,6 +118,9 @@ int tl_set_hgemm_k_rotation(int per_tile, int per_xcd);
 /* Tuning hook: the MFMA GEMM numbers its tiles down bands of `band` rows of tiles (0 = automatic; a value of
  * at least the number of tile rows numbers them down whole columns). */
 int tl_set_hgemm_tile_band(int band);
+/* Tuning hook: the kernel for 2 <= M <= 32 that keeps X in registers and streams W once (0 = automatic, -1 = never:
+ * such shapes then take the tile kernels). */
+int tl_set_hgemm_fewrows(int mode);
 /* Tuning hook: prefill attention kernel, 0 = automatic, 1 = one wavefront per 32 query rows,
  * 2 = LDS-tiled workgroups of 128 query rows (head_dim 128, ldv covering the context rounded up to 64). */
 int tl_set_prefill_attention_variant(int variant);

@@ -65,6 +65,7 @@ _PROTOS = {
     "tl_set_hgemm_splits": (_i, [_i]),
     "tl_set_hgemm_k_rotation": (_i, [_i, _i]),
     "tl_set_hgemm_tile_band": (_i, [_i]),
+    "tl_set_hgemm_fewrows": (_i, [_i]),
     "tl_set_prefill_attention_variant": (_i, [_i]),
     "tl_set_decode_attention_merge": (_i, [_i]),
     "tl_measure_mfma_rate_f16": (_i, [_i, _c.POINTER(_c.c_double)]),

@@ -837,6 +837,9 @@ static int launch_hgemm_cols(const void* A, const void* B, void* C, size_t M, si
         return TL_OK;
     }
     const int forced_variant = forced_vi ? forced_vi : g_forced_variant.load();
+    // a handful of rows and K up to 4096: X resident in registers, W streamed once, no split of K
+    if (forced_variant == 0 && g_forced_splits.load() == 0 && aligned16(C) && hgemm_fewrows_applies(M, N, K, ldc, batch))
+        return launch_hgemm_fewrows(A, B, C, M, N, K, ldc);
     int vi = forced_variant ? forced_variant : pick_variant(M, N, K, device_info().cu_count);
     if (g_variants[vi].stages > 0 && K % g_variants[vi].bk != 0) vi = 1;  // direct-to-LDS path cannot zero-fill a K tail
     // its per-lane byte offsets inside a tile ((rows - 1) * K + 64 halves) are 32-bit

@@ -85,6 +85,10 @@ int launch_hgemm(const void* A, const void* B, void* C, size_t M, size_t N, size
                  size_t sa, size_t sb, size_t sc, float** partials_out = nullptr, int* splits_out = nullptr,
                  Workspace::Lease* lease = nullptr);
 
+// Very few rows (2 <= M <= 32, K <= 4096): X stays in registers, W streams through once (hgemm_fewrows.hip).
+bool hgemm_fewrows_applies(size_t M, size_t N, size_t K, size_t ldc, size_t batch);
+int launch_hgemm_fewrows(const void* X, const void* W, void* C, size_t M, size_t N, size_t K, size_t ldc);
+
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
 #if defined(__HIPCC__)

@@ -243,6 +243,53 @@ def test_matmul2d_drawn_shapes_integer_exact(dev):
         assert np.array_equal(C.cpu().numpy().astype(np.float64), want), (i, M, N, K)
 
 
+FEW_ROWS_SHAPES = [(2, 16, 2048), (3, 48, 2304), (15, 4096, 4096), (16, 4112, 4096), (17, 1008, 3072), (31, 4096, 4096),
+                   (32, 11008, 4096), (8, 12288, 4096), (5, 32000, 4096), (32, 16384, 2560), (9, 272, 3840)]
+
+
+@pytest.mark.parametrize("shape", FEW_ROWS_SHAPES, ids=lambda s: "x".join(map(str, s)))
+def test_hgemm_few_rows_kernel(dev, oracle, shape):
+    """2 <= M <= 32 with K in 2048..4096 goes to the kernel that keeps X in registers and streams W once: every block
+    count per workgroup (fewer blocks than CUs, uneven shares), every row count around its 16-row groups, wavefronts
+    with 1 to 4 pieces of K.  Small integers are exact whatever the order of summation; random data is checked
+    against the oracle (all rows; sampled columns when W is large) and against the tile kernels."""
+    M, N, K = shape
+    A = synth.small_ints_f16(7300 + M, (M, K), -2, 2)
+    B = synth.small_ints_f16(7301 + N, (N, K), -2, 2)
+    C = torch.full((M, N), 5.0, device="cuda", dtype=torch.float16)
+    dev.hgemm(dev.from_numpy(A), dev.from_numpy(B), C)
+    want = A.astype(np.float64) @ B.astype(np.float64).T
+    assert np.abs(want).max() <= 2048
+    assert np.array_equal(C.cpu().numpy().astype(np.float64), want)
+
+    A = synth.normal_f16(7310 + M, (M, K), 1.0)
+    B = synth.normal_f16(7311 + N, (N, K), 0.02)
+    Ad, Bd = dev.from_numpy(A), dev.from_numpy(B)
+    got = dev.hgemm(Ad, Bd).cpu().numpy()
+    cols = np.arange(N) if N * K <= (1 << 24) else np.unique(np.random.default_rng(N).integers(0, N, 512))
+    ref = oracle.matmul2d(A, np.ascontiguousarray(B[cols]))
+    assert_close_f16(got[:, cols], ref, RTOL, ATOL, f"few-rows hgemm {shape}")
+    try:
+        dev.lib.tl_set_hgemm_fewrows(-1)
+        tiles = dev.hgemm(Ad, Bd).cpu().numpy()
+    finally:
+        dev.lib.tl_set_hgemm_fewrows(0)
+    assert_close_f16(got, tiles, RTOL, ATOL, f"few-rows hgemm vs tile kernels {shape}")
+
+
+def test_hgemm_few_rows_kernel_leaves_the_rest_of_c_alone(dev):
+    """The kernel stores 8-byte pieces of rows below M only: a C with more rows than M keeps them."""
+    M, N, K = 13, 4096, 4096
+    A = synth.small_ints_f16(7400, (M, K), -2, 2)
+    B = synth.small_ints_f16(7401, (N, K), -2, 2)
+    C = torch.full((M + 3, N), 5.0, device="cuda", dtype=torch.float16)
+    dev.hgemm(dev.from_numpy(A), dev.from_numpy(B), C[:M])
+    want = A.astype(np.float64) @ B.astype(np.float64).T
+    out = C.cpu().numpy().astype(np.float64)
+    assert np.array_equal(out[:M], want)
+    assert np.all(out[M:] == 5.0)
+
+
 def test_hgemm_k_rotation_and_splits_visit_every_k_tile_once(dev, oracle):
     """Workgroups start their walk over K at a rotated tile and wrap, per split: with small-integer data the
     result is exact whatever the order, so a skipped or repeated K tile shows as a wrong bit."""
