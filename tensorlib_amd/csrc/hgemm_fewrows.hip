@@ -5,7 +5,7 @@
 // With so few rows the product is a GEMV with a handful of right-hand sides: W has to stream from HBM once, and
 // nothing else should move.  A tile kernel cannot do that (its tiles re-read X through every CU and are padded to 128
 // rows), so this one is laid out like the GEMV:
-//   * a workgroup of four wavefronts owns 4096 values of K (wavefront w the 1024 from (4*group + w) * 1024) and
+//   * a workgroup of four wavefronts owns all of K (up to 4096: wavefront w the 1024 values from 1024 * w) and
 //     every parts-th 16-row block of W; each wavefront keeps ITS slice of X, all rows x 1024 values of K, in
 //     registers for the whole kernel, in the layout of the MFMA's second operand (MB x 128 registers per lane);
 //   * X first and then W stream through a ring private to the wavefront: a piece is 16 rows x 512 bytes, requested
