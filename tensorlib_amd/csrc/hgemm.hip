@@ -678,6 +678,8 @@ static const HgemmVariant g_variants[] = {
     // 192 columns: tile counts that fit 256 CUs where 128 and 256 columns do not (N = 11008, 12288)
     TL_HGEMM_PIPE(128, 192, 64, 4, 2, 4),  // 17
     TL_HGEMM_PIPE(256, 192, 64, 2, 2, 2),  // 18
+    // few rows: four wavefronts of 64x64 read a quarter fewer fragment bytes from LDS than eight of 64x32
+    TL_HGEMM_PIPE(128, 128, 64, 2, 2, 4),  // 19
 };
 
 static constexpr int kNumVariants = sizeof(g_variants) / sizeof(g_variants[0]);
@@ -715,7 +717,7 @@ static HgemmPlan plan_many_rows(size_t M, size_t N, size_t K, int cus) {
     static const int v_big = hgemm_variant_index("p256x256x64w2x4s2");
     static const int v_mid = hgemm_variant_index("p128x256x64w2x4s3");
     static const int v_small = hgemm_variant_index("p128x128x64w2x4s2");
-    static const int v_few_128x128 = hgemm_variant_index("p128x128x64w2x4s4");
+    static const int v_few_128x128 = hgemm_variant_index("p128x128x64w2x2s4");
     static const int v_256x192 = hgemm_variant_index("p256x192x64w2x2s2");
     auto tiles = [&](int bm, int bn) { return ((M + bm - 1) / bm) * ((N + bn - 1) / bn); };
     auto cost = [&](size_t t, size_t slots, double round_cost) {
@@ -753,7 +755,7 @@ static int pick_variant(size_t M, size_t N, size_t K, int cus) {
     static const int v_big = hgemm_variant_index("p256x256x64w2x4s2");
     static const int v_mid = hgemm_variant_index("p128x256x64w2x4s3");
     static const int v_few_256x128 = hgemm_variant_index("p256x128x64w2x4s3");
-    static const int v_few_128x128 = hgemm_variant_index("p128x128x64w2x4s4");
+    static const int v_few_128x128 = hgemm_variant_index("p128x128x64w2x2s4");
     static const int v_few_128x64 = hgemm_variant_index("p128x64x64w4x1s4");
     static const int v_few_128x192 = hgemm_variant_index("p128x192x64w4x2s4");
     auto tiles = [&](int bm, int bn) { return ((M + bm - 1) / bm) * ((N + bn - 1) / bn); };
@@ -764,7 +766,12 @@ static int pick_variant(size_t M, size_t N, size_t K, int cus) {
         if (M > 128 && tiles(128, 192) >= enough && tiles(128, 192) <= (size_t)cus) return v_few_128x192;
         if (M > 128 && tiles(128, 256) >= enough) return v_mid;   // measured ahead of 256x128 at equal tile counts
         if (M > 128 && tiles(256, 128) >= enough) return v_few_256x128;
-        // a long K can be halved instead of narrowing the tile
+        // A long K is split instead of narrowing the tile: wider tiles pull fewer bytes through a CU per output, and
+        // the slabs are small next to W (256x4096x11008: 128x128 tiles on four splits 40-43 us, 128x64 on two 48-49 us;
+        // 384 and 512 rows: 128x256 on four splits 54 and 62 us against 61 and 65 us).  With fewer than 256 rows the
+        // second row of 128-row tiles is mostly padding and the narrow tile stays ahead.
+        if (K >= 8192 && M >= 256 && tiles(128, 256) * 4 >= enough) return v_mid;
+        if (K >= 8192 && M >= 256 && tiles(128, 128) * 4 >= enough) return v_few_128x128;
         if (tiles(128, 128) >= enough || (K >= 8192 && tiles(128, 128) * 2 >= enough)) return v_few_128x128;
         return v_few_128x64;
     }
