@@ -712,8 +712,13 @@ struct HgemmPlan {
     int variant;
     double cost;
 };
-static HgemmPlan plan_many_rows(size_t M, size_t N, size_t K, int cus) {
-    (void)K;
+// more than 512 rows, few 128x256 tiles and a long K: split K instead of narrowing the tile
+static bool hgemm_many_rows_split(size_t M, size_t N, size_t K, int cus) {
+    const size_t t = ((M + 127) / 128) * ((N + 255) / 256);
+    return M > 512 && K >= 8192 && t * 2 <= (size_t)cus && t * 22016 <= (size_t)cus * K;
+}
+
+static HgemmPlan plan_many_rows(size_t M, size_t N, size_t K, int cus, bool can_split) {
     static const int v_big = hgemm_variant_index("p256x256x64w2x4s2");
     static const int v_mid = hgemm_variant_index("p128x256x64w2x4s3");
     static const int v_small = hgemm_variant_index("p128x128x64w2x4s2");
@@ -725,8 +730,14 @@ static HgemmPlan plan_many_rows(size_t M, size_t N, size_t K, int cus) {
         return round_cost * ((double)full + (rem ? 0.65 + 0.3 * (double)rem / (double)slots : 0.0));
     };
     const double c_small = cost(tiles(128, 128), (size_t)cus * 2, 0.66);
-    // a problem that leaves half the CUs without a 128x256 tile spreads wider as 128x128 tiles
-    if (tiles(128, 256) * 2 <= (size_t)cus) return {v_few_128x128, c_small};
+    // A problem that leaves half the CUs without a 128x256 tile: with a long K the tile stays and K is split over
+    // two to four workgroups (launch_hgemm_cols), as long as a split keeps about 2700 values of K (640x4096x11008:
+    // 72 against 103 us, 896x4096x11008: 97 against 103 us, 640x4096x8192: 57 against 67 us; from 1024x4096x11008
+    // and 896x4096x8192 on the slabs cost what the split wins); otherwise it spreads wider as 128x128 tiles.
+    if (tiles(128, 256) * 2 <= (size_t)cus) {
+        if (can_split && hgemm_many_rows_split(M, N, K, cus)) return {v_mid, c_small};
+        return {v_few_128x128, c_small};
+    }
     const double c_big = cost(tiles(256, 256), (size_t)cus, 1.0);
     const double c_mid = cost(tiles(128, 256), (size_t)cus, 0.613);
     const double c_192 = cost(tiles(256, 192), (size_t)cus, 0.865);   // three quarters of the work at 0.865 of the cost
@@ -751,7 +762,7 @@ static HgemmPlan plan_many_rows(size_t M, size_t N, size_t K, int cus) {
 // What does pay when whole rounds of 256x256 tiles are followed by a mostly empty one: launch the whole rounds as one
 // column range of C and the remaining columns as a second launch with whatever tiles suit THAT problem
 // (launch_hgemm; 2048x11008x4096: 344 big tiles = one round + 88 tiles, or one round + 176 tiles of 128x256).
-static int pick_variant(size_t M, size_t N, size_t K, int cus) {
+static int pick_variant(size_t M, size_t N, size_t K, int cus, bool can_split) {
     static const int v_big = hgemm_variant_index("p256x256x64w2x4s2");
     static const int v_mid = hgemm_variant_index("p128x256x64w2x4s3");
     static const int v_few_256x128 = hgemm_variant_index("p256x128x64w2x4s3");
@@ -770,12 +781,12 @@ static int pick_variant(size_t M, size_t N, size_t K, int cus) {
         // the slabs are small next to W (256x4096x11008: 128x128 tiles on four splits 40-43 us, 128x64 on two 48-49 us;
         // 384 and 512 rows: 128x256 on four splits 54 and 62 us against 61 and 65 us).  With fewer than 256 rows the
         // second row of 128-row tiles is mostly padding and the narrow tile stays ahead.
-        if (K >= 8192 && M >= 256 && tiles(128, 256) * 4 >= enough) return v_mid;
-        if (K >= 8192 && M >= 256 && tiles(128, 128) * 4 >= enough) return v_few_128x128;
+        if (can_split && K >= 8192 && M >= 256 && tiles(128, 256) * 4 >= enough) return v_mid;
+        if (can_split && K >= 8192 && M >= 256 && tiles(128, 128) * 4 >= enough) return v_few_128x128;
         if (tiles(128, 128) >= enough || (K >= 8192 && tiles(128, 128) * 2 >= enough)) return v_few_128x128;
         return v_few_128x64;
     }
-    return plan_many_rows(M, N, K, cus).variant;
+    return plan_many_rows(M, N, K, cus, can_split).variant;
 }
 
 // One launch (plus the ordered reduce when K is split) for columns [0, N) of a C whose rows are ldc elements apart.
@@ -799,9 +810,9 @@ int launch_hgemm(const void* A, const void* B, void* C, size_t M, size_t N, size
             const size_t full = col_tiles / cols_per_round, rem = col_tiles % cols_per_round;
             if (full >= 1 && rem > 0) {
                 const size_t N1 = full * cols_per_round * 256;
-                const double whole = plan_many_rows(M, N, K, cus).cost;
+                const double whole = plan_many_rows(M, N, K, cus, true).cost;
                 const double split = (double)full * (double)(tiles_m * cols_per_round) / (double)cus +
-                                     plan_many_rows(M, N - N1, K, cus).cost + 0.04;   // 0.04: the second launch's ramp
+                                     plan_many_rows(M, N - N1, K, cus, false).cost + 0.04;   // 0.04: the second launch's ramp
                 if (split < whole * 0.97) {
                     int rc = launch_hgemm_cols(A, B, C, M, N1, K, N, 1, 0, 0, 0, nullptr, nullptr, nullptr, v_big);
                     if (rc != TL_OK) return rc;
@@ -847,7 +858,8 @@ static int launch_hgemm_cols(const void* A, const void* B, void* C, size_t M, si
     // a handful of rows and K up to 4096: X resident in registers, W streamed once, no split of K
     if (forced_variant == 0 && g_forced_splits.load() == 0 && aligned16(C) && hgemm_fewrows_applies(M, N, K, ldc, batch))
         return launch_hgemm_fewrows(A, B, C, M, N, K, ldc);
-    int vi = forced_variant ? forced_variant : pick_variant(M, N, K, device_info().cu_count);
+    const bool can_split = batch == 1 && ldc == N;   // the second pass of a split K writes a dense C
+    int vi = forced_variant ? forced_variant : pick_variant(M, N, K, device_info().cu_count, can_split);
     if (g_variants[vi].stages > 0 && K % g_variants[vi].bk != 0) vi = 1;  // direct-to-LDS path cannot zero-fill a K tail
     // its per-lane byte offsets inside a tile ((rows - 1) * K + 64 halves) are 32-bit
     if (g_variants[vi].stages > 0 && K > ((size_t)1 << 22)) vi = 1;
@@ -892,6 +904,10 @@ static int launch_hgemm_cols(const void* A, const void* B, void* C, size_t M, si
             // (only for few rows: with more than 512 rows pick_variant already found a tile shape that
             // fills the chip well enough, and splitting measured slower there)
             splits = M <= 512 ? (int)((size_t)cus / nblocks) : 1;
+            if (M > 512 && forced_variant == 0 && can_split && hgemm_many_rows_split(M, N, K, cus)) {
+                splits = (int)((size_t)cus / nblocks);
+                if (splits > 4) splits = 4;
+            }
             const int max_by_k = KT / 8 > 0 ? KT / 8 : 1;
             if (splits > max_by_k) splits = max_by_k;
             if (splits > 16) splits = 16;

@@ -290,6 +290,37 @@ def test_hgemm_few_rows_kernel_leaves_the_rest_of_c_alone(dev):
     assert np.all(out[M:] == 5.0)
 
 
+@pytest.mark.parametrize("shape", [(640, 512, 8192), (576, 1280, 11008), (384, 1024, 8192), (256, 768, 11008)],
+                         ids=lambda s: "x".join(map(str, s)))
+def test_hgemm_long_k_is_split_over_wide_tiles(dev, shape):
+    """Few tiles and a long K: the dispatch keeps wide tiles and splits K over workgroups (fp32 slabs, ordered second
+    pass), also above 512 rows.  Small integers are exact whatever the split; the fused projection + add + RMSNorm entry
+    consumes the same slabs and must give the bits of the two-step path."""
+    M, N, K = shape
+    A = synth.small_ints_f16(7500 + M, (M, K), -2, 2)
+    B = synth.small_ints_f16(7501 + N, (N, K), -1, 1)
+    Ad, Bd = dev.from_numpy(A), dev.from_numpy(B)
+    C = dev.hgemm(Ad, Bd).cpu().numpy()
+    want = A.astype(np.float64) @ B.astype(np.float64).T
+    assert np.abs(want).max() <= 2048
+    assert np.array_equal(C.astype(np.float64), want)
+
+    A = synth.normal_f16(7510 + M, (M, K), 1.0)
+    B = synth.normal_f16(7511 + N, (N, K), 0.02)
+    R = synth.normal_f16(7512 + M, (M, N), 1.0)
+    g = synth.normal_f16(7513 + N, (N,), 1.0)
+    Ad, Bd, Rd, gd = (dev.from_numpy(x) for x in (A, B, R, g))
+    s1, n1 = dev.hgemm_add_rms_norm(Ad, Bd, Rd, gd, 1e-5)
+    P = dev.hgemm(Ad, Bd)
+    s2, n2 = dev.add_rms_norm(P, Rd, gd, 1e-5)
+    # the fused entry sums the slabs in fp32 and adds the residual before the one rounding of the sum, the two-step
+    # path rounds the product first: they agree to an ulp of the sum, and the plain product must match float64
+    ref = A.astype(np.float64) @ B.astype(np.float64).T
+    assert_close_f16(P.cpu().numpy(), ref.astype(np.float16), RTOL, ATOL, f"split long-K hgemm {shape}")
+    assert_close_f16(s1.cpu().numpy(), (ref + R.astype(np.float64)).astype(np.float16), RTOL, ATOL, f"fused sum {shape}")
+    assert_close_f16(s1.cpu().numpy(), s2.cpu().numpy(), RTOL, 2e-3, f"fused vs two-step sum {shape}")
+
+
 def test_hgemm_k_rotation_and_splits_visit_every_k_tile_once(dev, oracle):
     """Workgroups start their walk over K at a rotated tile and wrap, per split: with small-integer data the
     result is exact whatever the order, so a skipped or repeated K tile shows as a wrong bit."""
