@@ -112,6 +112,9 @@ const char* tl_hgemm_variant_name(int variant);
 int tl_measure_mfma_rate_f16(int mode, double* tflops);
 /* Tuning hook: force the number of K splits of the MFMA GEMM (0 = automatic). */
 int tl_set_hgemm_splits(int splits);
+/* Inspection hook (no reference counterpart): the kernel variant (index into tl_hgemm_variant_name(); -1 = the
+ * kernel for at most 32 rows) and the number of K splits the most recent fp16 GEMM launch of this process used. */
+int tl_hgemm_last_plan(int* variant, int* splits);
 /* Tuning hook: the MFMA GEMM's workgroups start their walk over K at K tile
  * (tile_column * per_tile + xcd * per_xcd) % tiles and wrap (-1 = automatic, 0 = no rotation). */
 int tl_set_hgemm_k_rotation(int per_tile, int per_xcd);

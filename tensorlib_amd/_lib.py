@@ -63,6 +63,7 @@ _PROTOS = {
     "tl_hgemm_variant_name": (_c.c_char_p, [_i]),
     "tl_set_gemv_grid_waves_per_cu": (_i, [_i]),
     "tl_set_hgemm_splits": (_i, [_i]),
+    "tl_hgemm_last_plan": (_i, [_c.POINTER(_c.c_int), _c.POINTER(_c.c_int)]),
     "tl_set_hgemm_k_rotation": (_i, [_i, _i]),
     "tl_set_hgemm_tile_band": (_i, [_i]),
     "tl_set_hgemm_fewrows": (_i, [_i]),

@@ -688,6 +688,7 @@ static std::atomic<int> g_forced_variant{0};
 static std::atomic<bool> g_attr_set[kNumVariants];
 
 static std::atomic<int> g_forced_splits{0};  // 0 = automatic
+static std::atomic<int> g_last_variant{0}, g_last_splits{0};   // what the most recent tile launch used
 static std::atomic<int> g_forced_rot_tile{-1}, g_forced_rot_xcd{-1};  // -1 = automatic
 static std::atomic<int> g_forced_band{0};                              // 0 = automatic
 
@@ -762,6 +763,32 @@ static HgemmPlan plan_many_rows(size_t M, size_t N, size_t K, int cus, bool can_
 // What does pay when whole rounds of 256x256 tiles are followed by a mostly empty one: launch the whole rounds as one
 // column range of C and the remaining columns as a second launch with whatever tiles suit THAT problem
 // (launch_hgemm; 2048x11008x4096: 344 big tiles = one round + 88 tiles, or one round + 176 tiles of 128x256).
+// Up to 512 rows and from 5120 columns on, 128x128 tiles on four wavefronts, split over K until they fill one round
+// of the chip, are as fast as or faster than the rules of pick_variant wherever they fill at least 70 % of the
+// compute units (60 % from 192 rows on) with K loops of 1024 to 8192 (sweep of seven tile shapes x six split counts over 152 shapes,
+// M = 48 .. 512, projections of Llama-size models 2048 to 8192 wide: 256x8192x8192 71.6 -> 52.8 us, 384x6144x4096
+// 52.1 -> 37.7, 256x5120x5120 38.0 -> 29.7, 48x11008x4096 26.1 -> 23.3; never more than 5 % slower).  With few rows
+// the kernel is bound by HBM long before the K loop of one workgroup is: then the smallest split whose K loop
+// (0.53 us per K tile of 64, less for a partly filled row tile) stays below the time HBM needs for W is enough, and
+// every further split only adds slabs.  Returns the number of splits, 0 when the rule does not apply.
+static int square_tile_splits(size_t M, size_t N, size_t K, int cus, bool can_split) {
+    if (M > 512 || N < 5120 || K % 64 != 0) return 0;
+    const size_t t = ((M + 127) / 128) * ((N + 127) / 128);
+    if (t > (size_t)cus) return 0;
+    const double hbm_us = (double)(N + M) * K * 2.0 / 5.5e6;
+    const double per_k_us = M < 128 ? 0.53 * (0.69 * M + 0.31 * 128 + 128) / 256 : 0.53;
+    const size_t KT = K / 64;
+    int sp = 1;
+    for (int s : {1, 2, 3, 4, 6}) {
+        if (t * s > (size_t)cus) break;
+        if (s > 1 && (!can_split || K < 4096 || K < (size_t)s * 1024)) break;
+        sp = s;
+        if ((double)((KT + s - 1) / s) * per_k_us <= hbm_us) break;
+    }
+    if (K > (size_t)sp * 8192 || t * sp * 10 < (size_t)cus * (M >= 192 ? 6 : 7)) return 0;
+    return sp;
+}
+
 static int pick_variant(size_t M, size_t N, size_t K, int cus, bool can_split) {
     static const int v_big = hgemm_variant_index("p256x256x64w2x4s2");
     static const int v_mid = hgemm_variant_index("p128x256x64w2x4s3");
@@ -774,7 +801,9 @@ static int pick_variant(size_t M, size_t N, size_t K, int cus, bool can_split) {
         const size_t enough = (size_t)cus * 6 / 10;
         if (tiles(256, 256) >= enough) return v_big;
         // one round either way: 192 columns put more CUs to work than 256 (512x12288x4096: 58 vs 65 us)
-        if (M > 128 && tiles(128, 192) >= enough && tiles(128, 192) <= (size_t)cus) return v_few_128x192;
+        // (not with a very long K that two splits of 128x256 tiles cover in one round: 512x8192x28672 319 -> 237 us)
+        const bool split_wide = can_split && K >= 16384 && M >= 256 && tiles(128, 256) * 2 <= (size_t)cus;
+        if (M > 128 && tiles(128, 192) >= enough && tiles(128, 192) <= (size_t)cus && !split_wide) return v_few_128x192;
         if (M > 128 && tiles(128, 256) >= enough) return v_mid;   // measured ahead of 256x128 at equal tile counts
         if (M > 128 && tiles(256, 128) >= enough) return v_few_256x128;
         // A long K is split instead of narrowing the tile: wider tiles pull fewer bytes through a CU per output, and
@@ -784,6 +813,8 @@ static int pick_variant(size_t M, size_t N, size_t K, int cus, bool can_split) {
         if (can_split && K >= 8192 && M >= 256 && tiles(128, 256) * 4 >= enough) return v_mid;
         if (can_split && K >= 8192 && M >= 256 && tiles(128, 128) * 4 >= enough) return v_few_128x128;
         if (tiles(128, 128) >= enough || (K >= 8192 && tiles(128, 128) * 2 >= enough)) return v_few_128x128;
+        // two rounds of narrow tiles lose to one partly filled round of square ones (384x6144x4096: 52 -> 38 us)
+        if (tiles(128, 64) > (size_t)cus) return v_few_128x128;
         return v_few_128x64;
     }
     return plan_many_rows(M, N, K, cus, can_split).variant;
@@ -856,10 +887,18 @@ static int launch_hgemm_cols(const void* A, const void* B, void* C, size_t M, si
     }
     const int forced_variant = forced_vi ? forced_vi : g_forced_variant.load();
     // a handful of rows and K up to 4096: X resident in registers, W streamed once, no split of K
-    if (forced_variant == 0 && g_forced_splits.load() == 0 && aligned16(C) && hgemm_fewrows_applies(M, N, K, ldc, batch))
+    if (forced_variant == 0 && g_forced_splits.load() == 0 && aligned16(C) && hgemm_fewrows_applies(M, N, K, ldc, batch)) {
+        g_last_variant = -1;
+        g_last_splits = 1;
         return launch_hgemm_fewrows(A, B, C, M, N, K, ldc);
+    }
     const bool can_split = batch == 1 && ldc == N;   // the second pass of a split K writes a dense C
     int vi = forced_variant ? forced_variant : pick_variant(M, N, K, device_info().cu_count, can_split);
+    int model_splits = 0;
+    if (forced_variant == 0 && g_forced_splits.load() == 0) {
+        model_splits = square_tile_splits(M, N, K, device_info().cu_count, can_split);
+        if (model_splits > 0) vi = hgemm_variant_index("p128x128x64w2x2s4");
+    }
     if (g_variants[vi].stages > 0 && K % g_variants[vi].bk != 0) vi = 1;  // direct-to-LDS path cannot zero-fill a K tail
     // its per-lane byte offsets inside a tile ((rows - 1) * K + 64 halves) are 32-bit
     if (g_variants[vi].stages > 0 && K > ((size_t)1 << 22)) vi = 1;
@@ -904,6 +943,7 @@ static int launch_hgemm_cols(const void* A, const void* B, void* C, size_t M, si
             // (only for few rows: with more than 512 rows pick_variant already found a tile shape that
             // fills the chip well enough, and splitting measured slower there)
             splits = M <= 512 ? (int)((size_t)cus / nblocks) : 1;
+            if (model_splits > 0) splits = model_splits;
             if (M > 512 && forced_variant == 0 && can_split && hgemm_many_rows_split(M, N, K, cus)) {
                 splits = (int)((size_t)cus / nblocks);
                 if (splits > 4) splits = 4;
@@ -923,6 +963,8 @@ static int launch_hgemm_cols(const void* A, const void* B, void* C, size_t M, si
             a.partial = lease.ptr;
         }
     }
+    g_last_variant = vi;
+    g_last_splits = splits;
     // pipelined kernels with up to three stages are persistent: one workgroup per resident slot walks several tiles
     size_t grid_x = nblocks;
     if (v.persistent) {
@@ -1025,6 +1067,13 @@ int tl_set_hgemm_k_rotation(int per_tile, int per_xcd) {
 int tl_set_hgemm_tile_band(int band) {
     TL_REQUIRE(band >= 0, "tl_set_hgemm_tile_band: negative band");
     tl::g_forced_band = band;
+    return TL_OK;
+}
+
+int tl_hgemm_last_plan(int* variant, int* splits) {
+    TL_REQUIRE(variant && splits, "tl_hgemm_last_plan: null output");
+    *variant = tl::g_last_variant.load();
+    *splits = tl::g_last_splits.load();
     return TL_OK;
 }
 

@@ -467,6 +467,15 @@ class HipDevice:
             out.append(n.decode())
             i += 1
 
+    def hgemm_last_plan(self) -> tuple[str, int]:
+        """(kernel variant, K splits) of the most recent fp16 GEMM launch; the variant of the kernel for at most
+        32 rows is reported as "fewrows"."""
+        import ctypes
+        v, s = ctypes.c_int(0), ctypes.c_int(0)
+        check(self.lib.tl_hgemm_last_plan(ctypes.byref(v), ctypes.byref(s)), "tl_hgemm_last_plan")
+        name = "fewrows" if v.value < 0 else self.lib.tl_hgemm_variant_name(v.value).decode()
+        return name, s.value
+
     def hgemm_variants(self) -> list[str]:
         out, i = [], 0
         while True:

@@ -321,6 +321,34 @@ def test_hgemm_long_k_is_split_over_wide_tiles(dev, shape):
     assert_close_f16(s1.cpu().numpy(), s2.cpu().numpy(), RTOL, 2e-3, f"fused vs two-step sum {shape}")
 
 
+SQUARE_TILE_PLANS = [
+    # (M, N, K), expected (variant, splits)
+    ((256, 8192, 8192), ("p128x128x64w2x2s4", 2)),
+    ((192, 5120, 5120), ("p128x128x64w2x2s4", 3)),
+    ((48, 12288, 4096), ("p128x128x64w2x2s4", 2)),
+    ((512, 8192, 2048), ("p128x128x64w2x2s4", 1)),
+    ((384, 6144, 4096), ("p128x128x64w2x2s4", 1)),   # two rounds of 128x64 tiles avoided
+    ((512, 8192, 16384), ("p128x256x64w2x4s3", 2)),  # very long K: wide tiles on two splits, not 128x192 unsplit
+    ((48, 4096, 4096), ("p128x64x64w4x1s4", 4)),     # fewer than 5120 columns: the narrow-tile rule stays
+    ((16, 4096, 4096), ("fewrows", 1)),
+]
+
+
+@pytest.mark.parametrize("shape,plan", SQUARE_TILE_PLANS, ids=lambda v: "x".join(map(str, v)) if isinstance(v[0], int) else None)
+def test_hgemm_square_tiles_fill_one_round(dev, shape, plan):
+    """Up to 512 rows and from 5120 columns on, 128x128 tiles are split over K until one round of them fills the chip.
+    The plan the dispatch took is read back through tl_hgemm_last_plan; small integers are exact whatever the plan."""
+    M, N, K = shape
+    A = synth.small_ints_f16(7600 + M, (M, K), -2, 2)
+    B = synth.small_ints_f16(7601 + N, (N, K), -1, 1)
+    Ad, Bd = dev.from_numpy(A), dev.from_numpy(B)
+    C = dev.hgemm(Ad, Bd)
+    assert dev.hgemm_last_plan() == plan
+    want = torch.from_numpy(A).cuda().double() @ torch.from_numpy(B).cuda().double().T
+    assert float(want.abs().max()) <= 2048
+    assert torch.equal(C.double(), want)
+
+
 def test_hgemm_k_rotation_and_splits_visit_every_k_tile_once(dev, oracle):
     """Workgroups start their walk over K at a rotated tile and wrap, per split: with small-integer data the
     result is exact whatever the order, so a skipped or repeated K tile shows as a wrong bit."""
