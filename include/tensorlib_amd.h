@@ -131,6 +131,9 @@ int tl_set_prefill_attention_variant(int variant);
  * up to 512 cached positions), 1 = always inside the launch, by the workgroup that finishes a head's last chunk,
  * 2 = always by a second launch.  Same bits either way. */
 int tl_set_decode_attention_merge(int mode);
+/* Tuning hook: cached positions per workgroup of the decode attention: 0 = automatic, else 64, 128 or 256
+ * (head_dim 256 always uses 64). */
+int tl_set_decode_attention_chunk(int positions);
 /* Tuning hook: cap the GEMV grid at `waves` resident wavefronts per compute unit (0 = default). */
 int tl_set_gemv_grid_waves_per_cu(int waves);
 
@@ -235,7 +238,8 @@ int tl_decode_attention_rope_f16(void* out, const void* qkv, void* cache_k, void
  * floats that is part of the library's code object (each GPU holds its copy until the process ends) instead of the
  * grown-on-demand workspace, and the call makes no hipMalloc / hipFree.  Limit:
  *   64 * ceil(n_heads / 64) + n_heads * ceil((pos + 1) / 64) * (head_dim + 2) <= TL_DECODE_ATTENTION_STATIC_SCRATCH_FLOATS
- * (32 heads of 128: 16128 positions); larger sizes return TL_EINVAL.  Every call on a GPU shares that GPU's array:
+ * (32 heads of 128: 16128 positions) is always accepted; what exceeds the array returns TL_EINVAL (contexts from 1280
+ * positions on with head_dim up to 128 are cut into chunks of 128 positions and need half of that).  Every call on a GPU shares that GPU's array:
  * calls that overlap on one GPU (two streams, two host threads) race; calls on one stream do not.  The caller clears
  * nothing: every partial a call reads was written by the same call, and the per-head tickets at the head of the array
  * (64 words per 64 heads, counted in the limit) are zero when the library is loaded and are set back to zero by the

@@ -69,6 +69,7 @@ _PROTOS = {
     "tl_set_hgemm_fewrows": (_i, [_i]),
     "tl_set_prefill_attention_variant": (_i, [_i]),
     "tl_set_decode_attention_merge": (_i, [_i]),
+    "tl_set_decode_attention_chunk": (_i, [_i]),
     "tl_measure_mfma_rate_f16": (_i, [_i, _c.POINTER(_c.c_double)]),
     "tl_rms_norm_f16": (_i, [_vp, _vp, _vp, _f, _i, _i]),
     "tl_apply_rotary_emb_f16": (_i, [_vp, _vp, _i, _i, _i, _i, _i]),

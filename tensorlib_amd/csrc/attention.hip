@@ -13,6 +13,7 @@
 // host-to-device copy per element.
 #include <atomic>
 #include <mutex>
+#include <type_traits>
 
 #include "tl_internal.h"
 
@@ -45,7 +46,9 @@ __device__ __forceinline__ float lanes_sum(float v) {
 }
 
 constexpr int kAttnThreads = 256;
-constexpr int kAttnChunk = 64;  // cached positions per workgroup
+constexpr int kAttnChunk = 64;  // cached positions per workgroup when a context is cut into many chunks
+// tuning hook: cached positions per workgroup, 0 = automatic, else 64, 128 or 256
+static std::atomic<int> g_decode_chunk{0};
 
 // partial layout per (head, chunk): [0] = max, [1] = sum, [2 .. 2+head_dim) = sum_t p_t * V[t]
 // Rotate the 4 (even, odd) pairs of one 16-byte chunk of a head vector; `d0` is the index of the
@@ -135,21 +138,23 @@ __device__ __forceinline__ void merge_head(half_t* out, const float* base, int h
 // the new v row into the caches (each head's workgroup writes only its own head slice).
 // ROPE: 0 = q is already rotated and the caches hold position T-1; 1 = rotate with the table's (cos, sin);
 // 2 = rotate with cos/sin evaluated in the kernel (no table given).
-template <int LPR, int ROPE>
+// CHUNK: cached positions per workgroup (64, 128 or 256; every thread holds CHUNK / GROUPS rows of K and of V).
+template <int LPR, int ROPE, int CHUNK>
 __global__ void __launch_bounds__(kAttnThreads)
 decode_attn_partial_kernel(half_t* out, float* partial, const half_t* q, half_t* cache_k,
                            half_t* cache_v, const half_t* rope_table, int T, int n_heads, float inv_scale,
                            int n_chunks, unsigned* tickets) {
     constexpr int D = LPR * 8;
     constexpr int GROUPS = kAttnThreads / LPR;
-    __shared__ float sc[kAttnChunk];
+    static_assert(CHUNK % 64 == 0 && CHUNK <= kAttnThreads && CHUNK % (kAttnThreads / LPR) == 0, "chunk size");
+    __shared__ float sc[CHUNK];
     __shared__ float red[16];
     __shared__ float obuf[GROUPS][D];
 
     const int h = blockIdx.x;
     const int chunk = blockIdx.y;
-    const int t0 = chunk * kAttnChunk;
-    const int t1 = (t0 + kAttnChunk < T) ? (t0 + kAttnChunk) : T;
+    const int t0 = chunk * CHUNK;
+    const int t1 = (t0 + CHUNK < T) ? (t0 + CHUNK) : T;
     const int tid = threadIdx.x;
     const int sub = tid % LPR;
     const int grp = tid / LPR;
@@ -167,7 +172,7 @@ decode_attn_partial_kernel(half_t* out, float* partial, const half_t* q, half_t*
 
     // All K and V rows this thread will touch are requested up front (NIT rows each), so the whole
     // kernel pays one global round trip instead of one per phase.
-    constexpr int NIT = kAttnChunk / GROUPS;
+    constexpr int NIT = CHUNK / GROUPS;
     half8_t kreg[NIT], vreg[NIT];
     const half8_t zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
     const size_t head_off = (size_t)h * D + sub * 8;
@@ -208,33 +213,60 @@ decode_attn_partial_kernel(half_t* out, float* partial, const half_t* q, half_t*
     }
     __syncthreads();
 
-    // chunk max and sum (kAttnChunk == 64: wavefront 0 alone can reduce it)
+    // chunk max and sum: thread t holds the score of position t0 + t; 64 positions are reduced by wavefront 0 alone,
+    // more by one wavefront per 64 and a second step over the wavefronts' results in ascending order
     float m, l;
     {
         const int n = t1 - t0;
         float v = (tid < n) ? sc[tid] : -INFINITY;
-        if (tid < 64) {
-            float mx = v;
-            mx = fmaxf(mx, dppf<0xB1>(mx));
-            mx = fmaxf(mx, dppf<0x4E>(mx));
-            mx = fmaxf(mx, dppf<0x141>(mx));
-            mx = fmaxf(mx, dppf<0x140>(mx));
-            mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-            mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+        auto wave_max = [](float x) {
+            x = fmaxf(x, dppf<0xB1>(x));
+            x = fmaxf(x, dppf<0x4E>(x));
+            x = fmaxf(x, dppf<0x141>(x));
+            x = fmaxf(x, dppf<0x140>(x));
+            x = fmaxf(x, __shfl_xor(x, 16, 64));
+            x = fmaxf(x, __shfl_xor(x, 32, 64));
+            return x;
+        };
+        auto wave_sum = [](float x) {
+            x += dppf<0xB1>(x);
+            x += dppf<0x4E>(x);
+            x += dppf<0x141>(x);
+            x += dppf<0x140>(x);
+            x += __shfl_xor(x, 16, 64);
+            x += __shfl_xor(x, 32, 64);
+            return x;
+        };
+        if constexpr (CHUNK == 64) {
+            if (tid < 64) {
+                const float mx = wave_max(v);
+                const float p = (tid < n) ? expf(v - mx) : 0.f;
+                const float sm = wave_sum(p);
+                if (tid < n) sc[tid] = p;
+                if (tid == 0) { red[0] = mx; red[1] = sm; }
+            }
+            __syncthreads();
+            m = red[0];
+            l = red[1];
+        } else {
+            constexpr int RW = CHUNK / 64;
+            const int wave = tid / 64;
+            float mx = wave_max(v);
+            if (tid % 64 == 0) red[wave] = mx;
+            __syncthreads();
+            mx = red[0];
+#pragma unroll
+            for (int w = 1; w < RW; ++w) mx = fmaxf(mx, red[w]);
             const float p = (tid < n) ? expf(v - mx) : 0.f;
-            float sm = p;
-            sm += dppf<0xB1>(sm);
-            sm += dppf<0x4E>(sm);
-            sm += dppf<0x141>(sm);
-            sm += dppf<0x140>(sm);
-            sm += __shfl_xor(sm, 16, 64);
-            sm += __shfl_xor(sm, 32, 64);
+            const float sm = wave_sum(p);
             if (tid < n) sc[tid] = p;
-            if (tid == 0) { red[0] = mx; red[1] = sm; }
+            if (tid % 64 == 0) red[8 + wave] = sm;
+            __syncthreads();
+            m = mx;
+            l = red[8];
+#pragma unroll
+            for (int w = 1; w < RW; ++w) l += red[8 + w];
         }
-        __syncthreads();
-        m = red[0];
-        l = red[1];
     }
 
     // weighted sum of V rows: thread (grp, sub) accumulates dims [sub*8, sub*8+8) over its positions
@@ -875,6 +907,21 @@ add_rms_norm_vec_kernel(half_t* sum_out, half_t* norm_out, const half_t* a, cons
     }
 }
 
+// Cached positions per workgroup of the decode attention.  Every launch boundary in a decode step costs about 3 us and
+// merging chunk partials another 2-2.5 us, so a context that one workgroup per head can hold in registers is not cut:
+// up to 128 positions one chunk of 128 (4.0-4.7 us against 5.5-5.8 us for two chunks of 64 merged in the kernel), up
+// to 192 one chunk of 256 (4.9-5.6 against 5.6-5.8 us).  Beyond that a single workgroup per head is bound by what one
+// CU takes in (256 positions: 6.2 us) and chunks of 64 over many CUs win again; from 1280 positions on chunks of 128
+// halve the partials the second launch merges (2048 positions: 10.0 against 11.5 us).  Times: one attention launch
+// between dependent 4096x4096 GEMVs, 32 heads of 128.
+static int decode_attention_chunk(int T, int head_dim) {
+    (void)head_dim;
+    if (T <= 64) return 64;
+    if (T <= 128) return 128;
+    if (T <= 192) return 256;
+    return T < 1280 ? 64 : 128;
+}
+
 // Library-owned fp32 workspace for the chunk partials, grown on demand.
 static Workspace g_partials;
 
@@ -926,7 +973,10 @@ static int launch_decode_attention(void* out, const void* q, void* cache_k, void
     TL_REQUIRE(tl::aligned16(q) && tl::aligned16(cache_k) && tl::aligned16(cache_v),
                "%s: q and the caches must be 16-byte aligned", name);
     TL_REQUIRE(n_heads <= 65535, "%s: too many heads", name);
-    const int n_chunks = (T + tl::kAttnChunk - 1) / tl::kAttnChunk;
+    int chunk = tl::g_decode_chunk.load();
+    if (chunk == 0) chunk = tl::decode_attention_chunk(T, head_dim);
+    if (head_dim == 256) chunk = tl::kAttnChunk;   // 32 rows of K and V per thread do not fit the registers
+    const int n_chunks = (T + chunk - 1) / chunk;
     TL_REQUIRE(n_chunks <= 65535, "%s: T=%d too long", name, T);
     tl::Workspace::Lease lease;   // held until both kernels are enqueued
     // [one ticket per head, padded to 64 words][partials]; tickets are zero between calls
@@ -935,9 +985,9 @@ static int launch_decode_attention(void* out, const void* q, void* cache_k, void
     float* ws = static_ws;
     if (static_ws) {
         TL_REQUIRE(ws_floats <= static_ws_floats,
-                   "%s: %d heads x %d chunks of 64 positions x (%d + 2) floats (+ tickets) = %zu floats of partial results exceed the "
+                   "%s: %d heads x %d chunks of %d positions x (%d + 2) floats (+ tickets) = %zu floats of partial results exceed the "
                    "static scratch of %zu floats; use tl_decode_attention_rope_f16 for this size",
-                   name, n_heads, n_chunks, head_dim, ws_floats, static_ws_floats);
+                   name, n_heads, n_chunks, chunk, head_dim, ws_floats, static_ws_floats);
     } else if (n_chunks > 1) {
         int rc = tl::g_partials.acquire(ws_floats, (size_t)1 << 20, "attention workspace", &lease);
         if (rc != TL_OK) return rc;
@@ -957,19 +1007,25 @@ static int launch_decode_attention(void* out, const void* q, void* cache_k, void
                            (const tl::half_t*)q, (tl::half_t*)cache_k, (tl::half_t*)cache_v,
                            (const tl::half_t*)rope_table, T, n_heads, inv_scale, n_chunks, tickets);
     };
-    if (fuse_rope && rope_table) {
-        if (head_dim == 64) launch(tl::decode_attn_partial_kernel<8, 1>);
-        else if (head_dim == 128) launch(tl::decode_attn_partial_kernel<16, 1>);
-        else launch(tl::decode_attn_partial_kernel<32, 1>);
-    } else if (fuse_rope) {
-        if (head_dim == 64) launch(tl::decode_attn_partial_kernel<8, 2>);
-        else if (head_dim == 128) launch(tl::decode_attn_partial_kernel<16, 2>);
-        else launch(tl::decode_attn_partial_kernel<32, 2>);
-    } else {
-        if (head_dim == 64) launch(tl::decode_attn_partial_kernel<8, 0>);
-        else if (head_dim == 128) launch(tl::decode_attn_partial_kernel<16, 0>);
-        else launch(tl::decode_attn_partial_kernel<32, 0>);
-    }
+    const int rope = fuse_rope ? (rope_table ? 1 : 2) : 0;
+    auto launch_chunk = [&](auto lpr, auto rp) {
+        constexpr int LPR = decltype(lpr)::value, RP = decltype(rp)::value;
+        if constexpr (LPR == 32) {
+            launch(tl::decode_attn_partial_kernel<LPR, RP, 64>);
+        } else {
+            if (chunk == 64) launch(tl::decode_attn_partial_kernel<LPR, RP, 64>);
+            else if (chunk == 128) launch(tl::decode_attn_partial_kernel<LPR, RP, 128>);
+            else launch(tl::decode_attn_partial_kernel<LPR, RP, 256>);
+        }
+    };
+    auto launch_rope = [&](auto lpr) {
+        if (rope == 0) launch_chunk(lpr, std::integral_constant<int, 0>{});
+        else if (rope == 1) launch_chunk(lpr, std::integral_constant<int, 1>{});
+        else launch_chunk(lpr, std::integral_constant<int, 2>{});
+    };
+    if (head_dim == 64) launch_rope(std::integral_constant<int, 8>{});
+    else if (head_dim == 128) launch_rope(std::integral_constant<int, 16>{});
+    else launch_rope(std::integral_constant<int, 32>{});
     TL_CHECK_LAUNCH("decode_attn_partial_kernel");
     if (n_chunks > 1 && !tickets) {
         hipLaunchKernelGGL(tl::decode_attn_merge_kernel, dim3(n_heads), dim3(256), 0, st, (tl::half_t*)out, partials, head_dim,
@@ -1004,6 +1060,13 @@ int tl_decode_attention_rope_static_f16(void* out, const void* qkv, void* cache_
     return launch_decode_attention(out, qkv, cache_k, cache_v, rope_table, pos + 1, n_heads, head_dim, true,
                                    "tl_decode_attention_rope_static_f16", ws,
                                    (size_t)TL_DECODE_ATTENTION_STATIC_SCRATCH_FLOATS);
+}
+
+int tl_set_decode_attention_chunk(int positions) {
+    TL_REQUIRE(positions == 0 || positions == 64 || positions == 128 || positions == 256,
+               "tl_set_decode_attention_chunk: %d is not 0, 64, 128 or 256", positions);
+    tl::g_decode_chunk = positions;
+    return TL_OK;
 }
 
 int tl_rope_table_f16(void* table, int max_seq, int head_dim) {

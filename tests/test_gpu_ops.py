@@ -180,7 +180,10 @@ def _attention_chain_oracle(oracle, q, ck, cv, T):
 
 
 @pytest.mark.parametrize("T,H,D", [(1, 32, 128), (5, 32, 128), (64, 32, 128), (65, 32, 128), (1024, 32, 128),
-                                   (2047, 32, 128), (300, 4, 64), (130, 2, 256)])
+                                   (2047, 32, 128), (300, 4, 64), (130, 2, 256),
+                                   # either side of every switch of the chunk size (64 / 128 / 256 positions per workgroup)
+                                   (128, 32, 128), (129, 32, 128), (192, 32, 128), (193, 32, 128), (1279, 8, 128),
+                                   (1280, 8, 128), (100, 4, 64), (190, 4, 64), (1300, 4, 64)])
 def test_decode_attention_fused_vs_chain(dev, oracle, T, H, D):
     S = max(T, 8)
     q = synth.normal_f16(90, (H, D), 1.0)
@@ -356,6 +359,29 @@ def test_rope_table_bits_equal_the_cpu_loop(dev, oracle, D):
     up to the handful of entries where the host libm is not correctly rounded (see rope_cos_sin_differences)."""
     differs = rope_cos_sin_differences(dev, oracle, 2048, D)
     assert differs.shape == (2048, D // 2) and not differs[0].any()
+
+
+@pytest.mark.parametrize("D", [64, 128])
+@pytest.mark.parametrize("chunk", [64, 128, 256])
+def test_decode_attention_every_chunk_size_vs_chain(dev, oracle, chunk, D):
+    """Each chunk size forced through the tuning hook, at contexts that end inside the first chunk, on a chunk boundary,
+    one past it, and in a partly filled last chunk of several."""
+    H = 6
+    q = synth.normal_f16(160, (H, D), 1.0)
+    ck = synth.normal_f16(161, (800, H, D), 1.0)
+    cv = synth.normal_f16(162, (800, H, D), 1.0)
+    qd, kd, vd = dev.from_numpy(q), dev.from_numpy(ck), dev.from_numpy(cv)
+    try:
+        dev.lib.tl_set_decode_attention_chunk(chunk)
+        for T in (1, chunk - 1, chunk, chunk + 1, 2 * chunk, 2 * chunk + 37, 800):
+            for mode in (1, 2):
+                dev.lib.tl_set_decode_attention_merge(mode)
+                got = dev.decode_attention(qd, kd, vd, T).cpu().numpy()
+                assert_close_f16(got, _attention_chain_oracle(oracle, q, ck, cv, T), RTOL, ATOL,
+                                 f"chunk {chunk} merge {mode} T={T}")
+    finally:
+        dev.lib.tl_set_decode_attention_chunk(0)
+        dev.lib.tl_set_decode_attention_merge(0)
 
 
 @pytest.mark.parametrize("T", [65, 200, 512, 513, 1500])
