@@ -349,6 +349,25 @@ def test_hgemm_square_tiles_fill_one_round(dev, shape, plan):
     assert torch.equal(C.double(), want)
 
 
+@pytest.mark.parametrize("shape", [(130, 5130, 4096), (257, 7000, 4160), (64, 8200, 8192), (500, 8100, 4096)],
+                         ids=lambda s: "x".join(map(str, s)))
+def test_hgemm_square_tiles_ragged_edges_and_batches(dev, shape):
+    """The same rule on shapes whose last tiles are partly filled, and as a batch of two (no split of K there: the
+    second pass of a split writes a dense single C)."""
+    M, N, K = shape
+    A = synth.small_ints_f16(7700 + M, (2, M, K), -2, 2)
+    B = synth.small_ints_f16(7701 + N, (N, K), -1, 1)
+    Ad, Bd = dev.from_numpy(A), dev.from_numpy(B)
+    want = torch.from_numpy(A).cuda().double() @ torch.from_numpy(B).cuda().double().T
+    assert float(want.abs().max()) <= 2048
+    C = dev.hgemm(Ad[0].contiguous(), Bd)
+    assert dev.hgemm_last_plan()[0] == "p128x128x64w2x2s4"
+    assert torch.equal(C.double(), want[0])
+    Cb = dev.matmul(Ad, Bd.t())
+    assert dev.hgemm_last_plan()[1] == 1
+    assert torch.equal(Cb.double(), want)
+
+
 def test_hgemm_k_rotation_and_splits_visit_every_k_tile_once(dev, oracle):
     """Workgroups start their walk over K at a rotated tile and wrap, per split: with small-integer data the
     result is exact whatever the order, so a skipped or repeated K tile shows as a wrong bit."""
