@@ -897,7 +897,8 @@ static int launch_hgemm_cols(const void* A, const void* B, void* C, size_t M, si
     int model_splits = 0;
     if (forced_variant == 0 && g_forced_splits.load() == 0) {
         model_splits = square_tile_splits(M, N, K, device_info().cu_count, can_split);
-        if (model_splits > 0) vi = hgemm_variant_index("p128x128x64w2x2s4");
+        static const int v_square = hgemm_variant_index("p128x128x64w2x2s4");
+        if (model_splits > 0) vi = v_square;
     }
     if (g_variants[vi].stages > 0 && K % g_variants[vi].bk != 0) vi = 1;  // direct-to-LDS path cannot zero-fill a K tail
     // its per-lane byte offsets inside a tile ((rows - 1) * K + 64 halves) are 32-bit

@@ -290,7 +290,8 @@ def test_hgemm_few_rows_kernel_leaves_the_rest_of_c_alone(dev):
     assert np.all(out[M:] == 5.0)
 
 
-@pytest.mark.parametrize("shape", [(640, 512, 8192), (576, 1280, 11008), (384, 1024, 8192), (256, 768, 11008)],
+@pytest.mark.parametrize("shape", [(640, 512, 8192), (576, 1280, 11008), (384, 1024, 8192), (256, 768, 11008),
+                                   (192, 5120, 5120), (64, 8192, 4096)],
                          ids=lambda s: "x".join(map(str, s)))
 def test_hgemm_long_k_is_split_over_wide_tiles(dev, shape):
     """Few tiles and a long K: the dispatch keeps wide tiles and splits K over workgroups (fp32 slabs, ordered second
