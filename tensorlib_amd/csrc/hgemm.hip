@@ -765,9 +765,10 @@ static HgemmPlan plan_many_rows(size_t M, size_t N, size_t K, int cus, bool can_
 // (launch_hgemm; 2048x11008x4096: 344 big tiles = one round + 88 tiles, or one round + 176 tiles of 128x256).
 // Up to 512 rows and from 5120 columns on, 128x128 tiles on four wavefronts, split over K until they fill one round
 // of the chip, are as fast as or faster than the rules of pick_variant wherever they fill at least 70 % of the
-// compute units (60 % from 192 rows on) with K loops of 1024 to 8192 (sweep of seven tile shapes x six split counts over 152 shapes,
-// M = 48 .. 512, projections of Llama-size models 2048 to 8192 wide: 256x8192x8192 71.6 -> 52.8 us, 384x6144x4096
-// 52.1 -> 37.7, 256x5120x5120 38.0 -> 29.7, 48x11008x4096 26.1 -> 23.3; never more than 5 % slower).  With few rows
+// compute units (60 % from 192 rows on) with K loops of 1024 to 8192 (sweep of seven tile shapes x six split counts
+// over 152 shapes, M = 48 .. 512, projections of Llama-size models 2048 to 8192 wide: 256x8192x8192 71.6 -> 52.8 us,
+// 384x6144x4096 52.1 -> 37.7, 256x5120x5120 38.0 -> 29.7, 48x12288x4096 26.8 -> 23.9; at most 5 % slower on the shapes
+// of that sweep it applies to).  With few rows
 // the kernel is bound by HBM long before the K loop of one workgroup is: then the smallest split whose K loop
 // (0.53 us per K tile of 64, less for a partly filled row tile) stays below the time HBM needs for W is enough, and
 // every further split only adds slabs.  Returns the number of splits, 0 when the rule does not apply.
@@ -894,11 +895,11 @@ static int launch_hgemm_cols(const void* A, const void* B, void* C, size_t M, si
     }
     const bool can_split = batch == 1 && ldc == N;   // the second pass of a split K writes a dense C
     int vi = forced_variant ? forced_variant : pick_variant(M, N, K, device_info().cu_count, can_split);
-    int model_splits = 0;
+    int square_splits = 0;
     if (forced_variant == 0 && g_forced_splits.load() == 0) {
-        model_splits = square_tile_splits(M, N, K, device_info().cu_count, can_split);
+        square_splits = square_tile_splits(M, N, K, device_info().cu_count, can_split);
         static const int v_square = hgemm_variant_index("p128x128x64w2x2s4");
-        if (model_splits > 0) vi = v_square;
+        if (square_splits > 0) vi = v_square;
     }
     if (g_variants[vi].stages > 0 && K % g_variants[vi].bk != 0) vi = 1;  // direct-to-LDS path cannot zero-fill a K tail
     // its per-lane byte offsets inside a tile ((rows - 1) * K + 64 halves) are 32-bit
@@ -944,7 +945,7 @@ static int launch_hgemm_cols(const void* A, const void* B, void* C, size_t M, si
             // (only for few rows: with more than 512 rows pick_variant already found a tile shape that
             // fills the chip well enough, and splitting measured slower there)
             splits = M <= 512 ? (int)((size_t)cus / nblocks) : 1;
-            if (model_splits > 0) splits = model_splits;
+            if (square_splits > 0) splits = square_splits;
             if (M > 512 && forced_variant == 0 && can_split && hgemm_many_rows_split(M, N, K, cus)) {
                 splits = (int)((size_t)cus / nblocks);
                 if (splits > 4) splits = 4;
