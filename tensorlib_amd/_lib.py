@@ -55,6 +55,7 @@ _PROTOS = {
     "tl_matmul2d_f16": (_i, [_vp, _vp, _vp, _sz, _sz, _sz]),
     "tl_gemv_f16": (_i, [_vp, _vp, _vp, _sz, _sz]),
     "tl_hgemm_f16": (_i, [_vp, _vp, _vp, _sz, _sz, _sz]),
+    "tl_hgemm_silu_mul_f16": (_i, [_vp, _vp, _vp, _vp, _sz, _sz, _sz]),
     "tl_matmul2d_batched_f16": (_i, [_vp, _vp, _vp, _sz, _sz, _sz, _sz, _sz, _sz, _sz]),
     "tl_matmul2d_f32": (_i, [_vp, _vp, _vp, _sz, _sz, _sz]),
     "tl_set_gemv_variant": (_i, [_i]),

@@ -44,6 +44,9 @@ struct HgemmArgs {
     int rot_tile, rot_xcd;
     // Tiles are numbered band by band: a band is band_m rows of tiles over all columns, walked column by column.
     int band_m;
+    // Gated launches (kernels built with MODE 2): B holds two matrices `gate` rows apart, N counts the rows of both
+    // (2 x the output columns), and C[m][n] = silu(A[m,:].B[n,:]) * (A[m,:].B[gate + n,:]) for n < N / 2.
+    int gate;
 };
 
 constexpr int kPad = 8;  // halves of padding per LDS row
@@ -215,6 +218,9 @@ __global__ void __launch_bounds__(WM* WN * 64) hgemm_f16_mfma_kernel(HgemmArgs a
 // Requirements: K % BK == 0 (no zero fill is possible on this path), K % 8 == 0, aligned operands.
 // MODE 0: every wavefront reads the fragments of a K step, then issues its MFMAs.
 // MODE 1: fragments double buffered in registers across K steps.
+// MODE 2: MODE 1 with the SwiGLU gate in the epilogue: a B tile holds, for every wavefront column, TN/2 rows of the
+//         first matrix followed by the TN/2 rows of the second that pair with them, so a wavefront finds both factors
+//         of an output in the 32 x TN block it stages through LDS anyway; the tile then covers BN/2 output columns.
 template <int BM, int BN, int BK, int WM, int WN, int STAGES, int MODE>
 __global__ void __launch_bounds__(WM* WN * 64) hgemm_f16_dlds_kernel(HgemmArgs a) {
     constexpr int NW = WM * WN;
@@ -230,6 +236,8 @@ __global__ void __launch_bounds__(WM* WN * 64) hgemm_f16_dlds_kernel(HgemmArgs a
     constexpr int TM = BM / WM, TN = BN / WN;
     constexpr int MT = TM / 32, NT = TN / 32;
     constexpr int KS = BK / 16;
+    constexpr bool GATED = MODE == 2;
+    static_assert(!GATED || TN % 16 == 0, "a wavefront column holds two halves of whole 16-byte pieces");
     static_assert(BK == 32 || BK == 64, "BK must be 32 or 64");
     static_assert(BM % (RPW * NW) == 0 && BN % (RPW * NW) == 0, "tile rows must split over the wavefronts");
     static_assert(STAGES >= 2 && STAGES <= 5 && LPW * (STAGES - 2) < 64, "vmcnt is a 6-bit counter");
@@ -238,7 +246,7 @@ __global__ void __launch_bounds__(WM* WN * 64) hgemm_f16_dlds_kernel(HgemmArgs a
     // one (staged through the last stage's LDS), so the C stores and the cold start of the next tile overlap.
     // vmcnt counts loads and stores together on this ISA, so the stores are drained (vmcnt(0)) before the
     // next tile's loop resumes waiting with exact load counts.
-    constexpr bool PERSIST = (STAGES <= 3 && MODE == 1 && NW * 32 * (BN / WN * 2 + 16) <= (BM + BN) * BK * 2);
+    constexpr bool PERSIST = (STAGES <= 3 && MODE >= 1 && NW * 32 * (BN / WN * 2 + 16) <= (BM + BN) * BK * 2);
 
     extern __shared__ __attribute__((aligned(1024))) unsigned char smem_raw[];
     typedef __attribute__((address_space(3))) unsigned char lds_byte_t;
@@ -263,7 +271,9 @@ __global__ void __launch_bounds__(WM* WN * 64) hgemm_f16_dlds_kernel(HgemmArgs a
     const int ldc = a.ldc;
     const unsigned rot_tile = (unsigned)a.rot_tile, rot_xcd = (unsigned)a.rot_xcd;
     const int band_m = a.band_m;
-    asm volatile("" ::"s"(partial), "s"(C), "s"(M), "s"(N), "s"(a.kt_per_split), "s"(rot_tile), "s"(rot_xcd), "s"(band_m), "s"(ldc));
+    const int gate = GATED ? a.gate : 0;
+    asm volatile("" ::"s"(partial), "s"(C), "s"(M), "s"(N), "s"(a.kt_per_split), "s"(rot_tile), "s"(rot_xcd), "s"(band_m), "s"(ldc),
+                 "s"(gate));
 
     // ---- loader: wavefront-load j of this wavefront covers tile rows (j*NW + wave)*RPW .. +RPW ----
     // A request's address is a wavefront-uniform base (first row of the tile at the K tile wanted, in scalar
@@ -284,10 +294,10 @@ __global__ void __launch_bounds__(WM* WN * 64) hgemm_f16_dlds_kernel(HgemmArgs a
         int tile_m, tile_n;
         tile_of_block(b, total_tiles, a.tiles_m, band_m, tile_m, tile_n);
         m0 = tile_m * BM;
-        n0 = tile_n * BN;
+        n0 = GATED ? tile_n * (BN / 2) : tile_n * BN;   // first output column of the tile
         rot = KT > 0 ? (int)(((unsigned)tile_n * rot_tile + (blockIdx.x & 7u) * rot_xcd) % (unsigned)KT) : 0;
         a_tile = A + (size_t)m0 * K + (size_t)kt_begin * BK;
-        b_tile = B + (size_t)n0 * K + (size_t)kt_begin * BK;
+        b_tile = GATED ? B + (size_t)kt_begin * BK : B + (size_t)n0 * K + (size_t)kt_begin * BK;
 #pragma unroll
         for (int j = 0; j < A_LOADS; ++j) {
             const int r = (j * NW + wave) * RPW + ld_row_in_group;  // tile row
@@ -299,8 +309,17 @@ __global__ void __launch_bounds__(WM* WN * 64) hgemm_f16_dlds_kernel(HgemmArgs a
         for (int j = 0; j < B_LOADS; ++j) {
             const int r = (j * NW + wave) * RPW + ld_row_in_group;
             const int c = ld_slot ^ ((r / RPL) % CPR);
-            const int rr = n0 + r < N ? r : N - 1 - n0;
-            b_voff[j] = (unsigned)(((size_t)rr * K + c * 8) * sizeof(half_t));
+            if constexpr (GATED) {
+                // tile row r = wavefront column r / TN, inside it TN/2 rows of the first matrix, then their partners;
+                // offsets are relative to B (the host checks that both matrices lie within 4 GB of it)
+                const int in_wave = r % TN;
+                const int ocol = n0 + (r / TN) * (TN / 2) + in_wave % (TN / 2);
+                const size_t grow = (size_t)(ocol < N / 2 ? ocol : N / 2 - 1) + (in_wave >= TN / 2 ? (size_t)gate : 0);
+                b_voff[j] = (unsigned)((grow * K + c * 8) * sizeof(half_t));
+            } else {
+                const int rr = n0 + r < N ? r : N - 1 - n0;
+                b_voff[j] = (unsigned)(((size_t)rr * K + c * 8) * sizeof(half_t));
+            }
         }
     };
     int vb = blockIdx.x;
@@ -387,7 +406,7 @@ __global__ void __launch_bounds__(WM* WN * 64) hgemm_f16_dlds_kernel(HgemmArgs a
 #pragma unroll
             for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
 
-    if constexpr (MODE == 1) {
+    if constexpr (MODE >= 1) {
         // Fragments are double buffered in registers: the ds_reads of K step s+1 (or of the next tile's first
         // step, after the tile barrier) go out one by one behind the first MFMAs of step s, in the order
         // load_frags uses.
@@ -491,9 +510,10 @@ __global__ void __launch_bounds__(WM* WN * 64) hgemm_f16_dlds_kernel(HgemmArgs a
     // ---- epilogue.  acc[i][j][4*g + r] = C[row i*32 + lane%32][col j*32 + 8*g + 4*(lane/32) + r] ----
     const int e_row = lane & 31;
     const int e_col = (lane >> 5) * 4;
-    const int row_base = m0 + wm * TM, col_base = n0 + wn * TN;
+    const int row_base = m0 + wm * TM, col_base = GATED ? n0 + wn * (TN / 2) : n0 + wn * TN;
     constexpr int RS = TN * 2 + 16;          // bytes per staged row of the fp16 epilogue
-    const bool staged = !partial && (N % 8) == 0 && (ldc % 8) == 0 && (reinterpret_cast<uintptr_t>(C) & 15u) == 0;
+    // (a gated launch is always staged: the host launches it only for 16-byte aligned rows of C and without split)
+    const bool staged = GATED || (!partial && (N % 8) == 0 && (ldc % 8) == 0 && (reinterpret_cast<uintptr_t>(C) & 15u) == 0);
     const int next_vb = vb + (int)gridDim.x;
     const bool has_next_tile = PERSIST && next_vb < total_tiles;
     if (staged || has_next_tile) {
@@ -513,7 +533,40 @@ __global__ void __launch_bounds__(WM* WN * 64) hgemm_f16_dlds_kernel(HgemmArgs a
             stage_area = (STAGES - 1) * STAGE_BYTES;
         }
     }
-    if (partial) {
+    if constexpr (GATED) {
+        // 32 x TN halves per block through the wavefront's LDS region as below; read back as pairs of 16-byte pieces
+        // TN/2 columns apart: out = half(silu(a) * b) of the two rounded projections, the arithmetic of SiluMulOp.
+        constexpr int TN2 = TN / 2, CHG = TN2 / 8, RPRG = 64 / CHG, PASSG = (32 + RPRG - 1) / RPRG;
+        static_assert(NW * 32 * RS <= STAGES * STAGE_BYTES, "staging area must fit the ring");
+        unsigned char* region = smem_raw + stage_area + wave * (32 * RS);
+        const int n_out = N / 2;
+#pragma unroll
+        for (int i = 0; i < MT; ++i) {
+#pragma unroll
+            for (int j = 0; j < NT; ++j)
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    half4_t h = {(half_t)acc[i][j][4 * g], (half_t)acc[i][j][4 * g + 1], (half_t)acc[i][j][4 * g + 2],
+                                 (half_t)acc[i][j][4 * g + 3]};
+                    *reinterpret_cast<half4_t*>(region + e_row * RS + (j * 32 + g * 8 + e_col) * 2) = h;
+                }
+#pragma unroll
+            for (int q = 0; q < PASSG; ++q) {
+                const int r = q * RPRG + lane / CHG, c = lane % CHG;
+                const int row = row_base + i * 32 + r, col = col_base + c * 8;
+                if (lane >= RPRG * CHG || r >= 32 || row >= M || col >= n_out) continue;
+                const half8_t va = *reinterpret_cast<const half8_t*>(region + r * RS + c * 16);
+                const half8_t vb = *reinterpret_cast<const half8_t*>(region + r * RS + TN2 * 2 + c * 16);
+                half8_t o;
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    const float x = (float)va[e];
+                    o[e] = (half_t)(x * (1.0f / (1.0f + expf(-x))) * (float)vb[e]);
+                }
+                *reinterpret_cast<half8_t*>(C + (size_t)row * ldc + col) = o;
+            }
+        }
+    } else if (partial) {
         // split-K: fp32 partial sums, four consecutive columns (16 bytes) per store where the row allows it
         const bool vec = (N % 4) == 0;
 #pragma unroll
@@ -642,20 +695,22 @@ struct HgemmVariant {
     int stages;  // 0: register-staged kernel (any K % 8 == 0); >= 2: direct-to-LDS ring (K % bk == 0)
     void (*kernel)(HgemmArgs);
     bool persistent;  // the kernel walks tiles blockIdx.x, + gridDim.x, ... (same predicate as PERSIST in the kernel)
+    void (*gated_kernel)(HgemmArgs);  // the same kernel with the SwiGLU gate in its epilogue (pipelined variants), else null
 };
 
 #define TL_HGEMM_VARIANT(BM, BN, BK, WM, WN) \
-    { "t" #BM "x" #BN "x" #BK "w" #WM "x" #WN, BM, BN, BK, WM * WN * 64, 0, hgemm_f16_mfma_kernel<BM, BN, BK, WM, WN>, false }
+    { "t" #BM "x" #BN "x" #BK "w" #WM "x" #WN, BM, BN, BK, WM * WN * 64, 0, hgemm_f16_mfma_kernel<BM, BN, BK, WM, WN>, false, nullptr }
 #define TL_HGEMM_DLDS(BM, BN, BK, WM, WN, ST) \
     { "d" #BM "x" #BN "x" #BK "w" #WM "x" #WN "s" #ST, BM, BN, BK, WM * WN * 64, ST, \
-      hgemm_f16_dlds_kernel<BM, BN, BK, WM, WN, ST, 0>, false }
+      hgemm_f16_dlds_kernel<BM, BN, BK, WM, WN, ST, 0>, false, nullptr }
 #define TL_HGEMM_PIPE(BM, BN, BK, WM, WN, ST) \
     { "p" #BM "x" #BN "x" #BK "w" #WM "x" #WN "s" #ST, BM, BN, BK, WM * WN * 64, ST, \
       hgemm_f16_dlds_kernel<BM, BN, BK, WM, WN, ST, 1>, \
-      (ST) <= 3 && (WM) * (WN) * 32 * ((BN) / (WN) * 2 + 16) <= ((BM) + (BN)) * (BK) * 2 }
+      (ST) <= 3 && (WM) * (WN) * 32 * ((BN) / (WN) * 2 + 16) <= ((BM) + (BN)) * (BK) * 2, \
+      hgemm_f16_dlds_kernel<BM, BN, BK, WM, WN, ST, 2> }
 
 static const HgemmVariant g_variants[] = {
-    {"auto", 0, 0, 0, 0, 0, nullptr, false},
+    {"auto", 0, 0, 0, 0, 0, nullptr, false, nullptr},
     // register-staged kernel: serves K % 64 != 0 (index 1 is the fallback of launch_hgemm)
     TL_HGEMM_VARIANT(128, 128, 64, 2, 2),  // 1
     TL_HGEMM_VARIANT(256, 256, 64, 2, 4),  // 2
@@ -685,7 +740,7 @@ static const HgemmVariant g_variants[] = {
 static constexpr int kNumVariants = sizeof(g_variants) / sizeof(g_variants[0]);
 // Tuning knobs (tests and sweeps set them, any thread may read them while launching).
 static std::atomic<int> g_forced_variant{0};
-static std::atomic<bool> g_attr_set[kNumVariants];
+static std::atomic<bool> g_attr_set[kNumVariants], g_attr_set_gated[kNumVariants];
 
 static std::atomic<int> g_forced_splits{0};  // 0 = automatic
 static std::atomic<int> g_last_variant{0}, g_last_splits{0};   // what the most recent tile launch used
@@ -823,12 +878,15 @@ static int pick_variant(size_t M, size_t N, size_t K, int cus, bool can_split) {
 
 // One launch (plus the ordered reduce when K is split) for columns [0, N) of a C whose rows are ldc elements apart.
 // forced_vi: 0 = dispatch by shape.
+// gate: 0, or the distance in rows between the two matrices stacked in B of a gated launch (HgemmArgs::gate); N then
+// counts the rows of both and C has N / 2 columns.
 static int launch_hgemm_cols(const void* A, const void* B, void* C, size_t M, size_t N, size_t K, size_t ldc, size_t batch,
                              size_t sa, size_t sb, size_t sc, float** partials_out, int* splits_out,
-                             Workspace::Lease* lease_out, int forced_vi);
+                             Workspace::Lease* lease_out, int forced_vi, size_t gate = 0);
 
 int launch_hgemm(const void* A, const void* B, void* C, size_t M, size_t N, size_t K, size_t batch, size_t sa,
-                 size_t sb, size_t sc, float** partials_out, int* splits_out, Workspace::Lease* lease_out) {
+                 size_t sb, size_t sc, float** partials_out, int* splits_out, Workspace::Lease* lease_out, size_t gate) {
+    const size_t ldc_all = gate ? N / 2 : N;   // row stride of C; a gated launch writes one column per pair of rows of B
     // Whole rounds of 256x256 tiles, then the remaining columns as a problem of their own, when the schedule model
     // says the two launches beat the best single one.  Only for many rows (no split-K there, so C is written
     // directly and a column range of it is just a pointer offset with the full row stride).
@@ -846,21 +904,22 @@ int launch_hgemm(const void* A, const void* B, void* C, size_t M, size_t N, size
                 const double split = (double)full * (double)(tiles_m * cols_per_round) / (double)cus +
                                      plan_many_rows(M, N - N1, K, cus, false).cost + 0.04;   // 0.04: the second launch's ramp
                 if (split < whole * 0.97) {
-                    int rc = launch_hgemm_cols(A, B, C, M, N1, K, N, 1, 0, 0, 0, nullptr, nullptr, nullptr, v_big);
+                    const size_t c1 = gate ? N1 / 2 : N1;   // first column of C (and row of B) of the second launch
+                    int rc = launch_hgemm_cols(A, B, C, M, N1, K, ldc_all, 1, 0, 0, 0, nullptr, nullptr, nullptr, v_big, gate);
                     if (rc != TL_OK) return rc;
                     if (splits_out) *splits_out = 1;
-                    return launch_hgemm_cols(A, (const half_t*)B + N1 * K, (half_t*)C + N1, M, N - N1, K, N, 1, 0, 0, 0,
-                                             nullptr, nullptr, nullptr, 0);
+                    return launch_hgemm_cols(A, (const half_t*)B + c1 * K, (half_t*)C + c1, M, N - N1, K, ldc_all, 1, 0, 0, 0,
+                                             nullptr, nullptr, nullptr, 0, gate);
                 }
             }
         }
     }
-    return launch_hgemm_cols(A, B, C, M, N, K, N, batch, sa, sb, sc, partials_out, splits_out, lease_out, 0);
+    return launch_hgemm_cols(A, B, C, M, N, K, ldc_all, batch, sa, sb, sc, partials_out, splits_out, lease_out, 0, gate);
 }
 
 static int launch_hgemm_cols(const void* A, const void* B, void* C, size_t M, size_t N, size_t K, size_t ldc, size_t batch,
                              size_t sa, size_t sb, size_t sc, float** partials_out, int* splits_out,
-                             Workspace::Lease* lease_out, int forced_vi) {
+                             Workspace::Lease* lease_out, int forced_vi, size_t gate) {
     Workspace::Lease own_lease;
     Workspace::Lease& lease = lease_out ? *lease_out : own_lease;
     if (splits_out) *splits_out = 1;
@@ -870,7 +929,7 @@ static int launch_hgemm_cols(const void* A, const void* B, void* C, size_t M, si
     hipStream_t st = stream();
     if (K == 0) {
         for (size_t b = 0; b < batch; ++b) {
-            int rc = launch_fill_f16((half_t*)C + b * sc, 0, M * N);
+            int rc = launch_fill_f16((half_t*)C + b * sc, 0, gate ? M * (N / 2) : M * N);
             if (rc != TL_OK) return rc;
         }
         return TL_OK;
@@ -878,6 +937,7 @@ static int launch_hgemm_cols(const void* A, const void* B, void* C, size_t M, si
     const bool vec_ok = (K % 8 == 0) && aligned16(A) && aligned16(B) &&
                         (batch == 1 || (sa % 8 == 0 && sb % 8 == 0));
     if (!vec_ok) {
+        TL_REQUIRE(gate == 0, "hgemm: a gated launch needs K %% 8 == 0 and 16-byte aligned operands");
         TL_REQUIRE(ldc == N, "hgemm generic path: a column range of C is not supported");
         dim3 grid((unsigned)((N + 15) / 16), (unsigned)((M + 15) / 16), (unsigned)batch);
         TL_REQUIRE(grid.y <= 65535, "hgemm generic path: M too large (%zu)", M);
@@ -888,7 +948,8 @@ static int launch_hgemm_cols(const void* A, const void* B, void* C, size_t M, si
     }
     const int forced_variant = forced_vi ? forced_vi : g_forced_variant.load();
     // a handful of rows and K up to 4096: X resident in registers, W streamed once, no split of K
-    if (forced_variant == 0 && g_forced_splits.load() == 0 && aligned16(C) && hgemm_fewrows_applies(M, N, K, ldc, batch)) {
+    if (gate == 0 && forced_variant == 0 && g_forced_splits.load() == 0 && aligned16(C) &&
+        hgemm_fewrows_applies(M, N, K, ldc, batch)) {
         g_last_variant = -1;
         g_last_splits = 1;
         return launch_hgemm_fewrows(A, B, C, M, N, K, ldc);
@@ -906,10 +967,20 @@ static int launch_hgemm_cols(const void* A, const void* B, void* C, size_t M, si
     if (g_variants[vi].stages > 0 && K > ((size_t)1 << 22)) vi = 1;
     const HgemmVariant& v = g_variants[vi];
     const size_t lds = lds_bytes(v);
-    if (lds > 64 * 1024 && !g_attr_set[vi].load()) {
-        TL_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(v.kernel),
+    void (*const kernel)(HgemmArgs) = gate ? v.gated_kernel : v.kernel;
+    if (gate) {
+        // what hgemm_gated_applies checks, once more where a violation would fault: the pipelined kernel, a C the
+        // staged epilogue can store to in 16-byte pieces, and 32-bit lane offsets that reach both matrices
+        TL_REQUIRE(kernel != nullptr && v.stages > 0, "hgemm: variant %s has no gated kernel", v.name);
+        TL_REQUIRE(batch == 1 && N % 16 == 0 && ldc % 8 == 0 && aligned16(C) && gate >= N / 2 &&
+                       (gate + N / 2) * K * sizeof(half_t) < ((size_t)1 << 32),
+                   "hgemm: gated launch outside its limits (N=%zu ldc=%zu gate=%zu K=%zu)", N, ldc, gate, K);
+    }
+    std::atomic<bool>& attr_set = gate ? g_attr_set_gated[vi] : g_attr_set[vi];
+    if (lds > 64 * 1024 && !attr_set.load()) {
+        TL_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-        g_attr_set[vi].store(true);
+        attr_set.store(true);
     }
     HgemmArgs a;
     a.A = (const half_t*)A;
@@ -930,6 +1001,7 @@ static int launch_hgemm_cols(const void* A, const void* B, void* C, size_t M, si
     a.partial = nullptr;
     a.rot_tile = 0;
     a.rot_xcd = 0;
+    a.gate = (int)gate;
     // band height that balances the panels of A and B an XCD's 32 tiles pull through its L2
     const int forced_band = g_forced_band.load();
     a.band_m = forced_band > 0 ? forced_band : (v.bm >= 2 * v.bn ? 4 : 8);
@@ -956,7 +1028,7 @@ static int launch_hgemm_cols(const void* A, const void* B, void* C, size_t M, si
             if (splits < 1) splits = 1;
         }
         if (splits > KT) splits = KT;
-        if (batch != 1 || ldc != N) splits = 1;   // the reduce pass writes a dense C
+        if (batch != 1 || ldc != N || gate) splits = 1;   // the reduce pass writes a dense C, and it does not gate
         if (splits > 1) {
             a.kt_per_split = (KT + splits - 1) / splits;
             splits = (KT + a.kt_per_split - 1) / a.kt_per_split;
@@ -987,7 +1059,7 @@ static int launch_hgemm_cols(const void* A, const void* B, void* C, size_t M, si
         if (rt >= 0) a.rot_tile = rt;
         if (rx >= 0) a.rot_xcd = rx;
     }
-    hipLaunchKernelGGL(v.kernel, dim3((unsigned)grid_x, (unsigned)batch, (unsigned)splits), dim3(v.threads), lds, st, a);
+    hipLaunchKernelGGL(kernel, dim3((unsigned)grid_x, (unsigned)batch, (unsigned)splits), dim3(v.threads), lds, st, a);
     TL_CHECK_LAUNCH(v.name);
     if (splits > 1 && partials_out && splits_out) {
         // the caller folds the second pass of split-K into its own kernel
@@ -1007,6 +1079,15 @@ static int launch_hgemm_cols(const void* A, const void* B, void* C, size_t M, si
     return TL_OK;
 }
 
+// One launch can apply the gate when the pipelined kernels serve the shape (K in whole tiles of 64, lane offsets within
+// 32 bits over both matrices), C takes 16-byte stores, and no variant without a gated build is forced.
+bool hgemm_gated_applies(const void* A, const void* B, const void* C, size_t M, size_t n_out, size_t K, size_t gate) {
+    const int forced = g_forced_variant.load();
+    return M >= 2 && n_out > 0 && n_out % 8 == 0 && gate >= n_out && K > 0 && K % 64 == 0 && K <= ((size_t)1 << 22) &&
+           M <= 0x7fffffffu && 2 * n_out <= 0x7fffffffu && (gate + n_out) * K * sizeof(half_t) < ((size_t)1 << 32) &&
+           aligned16(A) && aligned16(B) && aligned16(C) && (forced == 0 || g_variants[forced].gated_kernel != nullptr);
+}
+
 }  // namespace tl
 
 extern "C" {
@@ -1022,6 +1103,20 @@ int tl_matmul2d_f16(const void* A, const void* B, void* C, size_t M, size_t N, s
     TL_REQUIRE(A && B && C, "tl_matmul2d_f16: null pointer");
     if (M == 1) return tl::launch_gemv(A, B, C, N, K, 1, 0, 0, 0, 0);
     return tl::launch_hgemm(A, B, C, M, N, K, 1, 0, 0, 0);
+}
+
+int tl_hgemm_silu_mul_f16(const void* X, const void* W13, void* scratch, void* out, size_t M, size_t hidden, size_t K) {
+    TL_ENSURE_INIT();
+    if (M == 0 || hidden == 0) return TL_OK;
+    TL_REQUIRE(X && W13 && out, "tl_hgemm_silu_mul_f16: null pointer");
+    TL_REQUIRE(hidden % 8 == 0, "tl_hgemm_silu_mul_f16: hidden %% 8 != 0 (%zu)", hidden);
+    // a handful of rows: the kernel that keeps X in registers plus the separate gate is the faster pair
+    if (tl::hgemm_gated_applies(X, W13, out, M, hidden, K, hidden) && !tl::hgemm_fewrows_applies(M, 2 * hidden, K, 2 * hidden, 1))
+        return tl::launch_hgemm(X, W13, out, M, 2 * hidden, K, 1, 0, 0, 0, nullptr, nullptr, nullptr, hidden);
+    TL_REQUIRE(scratch, "tl_hgemm_silu_mul_f16: this shape takes the two-step path and needs the scratch buffer");
+    int rc = tl_matmul2d_f16(X, W13, scratch, M, 2 * hidden, K);
+    if (rc != TL_OK) return rc;
+    return tl_silu_mul_rows_f16(out, scratch, M, hidden);
 }
 
 int tl_matmul2d_batched_f16(const void* A, const void* B, void* C, size_t M, size_t N, size_t K, size_t batch,

@@ -83,7 +83,10 @@ int launch_gemv(const void* x, const void* W, void* y, size_t N, size_t K, size_
 // `lease` then keeps the slabs' buffer locked until the caller has enqueued its consumer.
 int launch_hgemm(const void* A, const void* B, void* C, size_t M, size_t N, size_t K, size_t batch,
                  size_t sa, size_t sb, size_t sc, float** partials_out = nullptr, int* splits_out = nullptr,
-                 Workspace::Lease* lease = nullptr);
+                 Workspace::Lease* lease = nullptr, size_t gate = 0);
+// gate != 0 (batch 1, no slabs): B stacks two matrices `gate` rows apart, N counts the rows of both, and
+// C[M, N/2] = silu(A.B1^T) * (A.B2^T), the gate applied in the GEMM's epilogue.  Only where hgemm_gated_applies() says so.
+bool hgemm_gated_applies(const void* A, const void* B, const void* C, size_t M, size_t n_out, size_t K, size_t gate);
 
 // Very few rows (2 <= M <= 32, K <= 4096): X stays in registers, W streams through once (hgemm_fewrows.hip).
 bool hgemm_fewrows_applies(size_t M, size_t N, size_t K, size_t ldc, size_t batch);

@@ -437,6 +437,22 @@ class HipDevice:
         check(self.lib.tl_silu_mul_rows_f16(_ptr(out), _ptr(ab), rows, two_h // 2), "tl_silu_mul_rows_f16")
         return out
 
+    def hgemm_silu_mul(self, X: torch.Tensor, W13: torch.Tensor, scratch: torch.Tensor | None = None) -> torch.Tensor:
+        """silu(X @ W1.T) * (X @ W3.T) for W13 = [W1; W3] of shape [2*hidden, K]; one launch where the pipelined GEMM
+        serves the shape, else GEMM into `scratch` ([M, 2*hidden], allocated here when not given) and the gate kernel."""
+        _req(X, name="X"), _req(W13, name="W13")
+        M, K = X.shape
+        two_h, K2 = W13.shape
+        if K != K2 or two_h % 2:
+            raise ValueError("Shape mismatch: X [M, K] against W13 [2*hidden, K]")
+        if scratch is None:
+            scratch = torch.empty((M, two_h), dtype=torch.float16, device=X.device)
+        _req(scratch, name="scratch")
+        out = torch.empty((M, two_h // 2), dtype=torch.float16, device=X.device)
+        check(self.lib.tl_hgemm_silu_mul_f16(_ptr(X), _ptr(W13), _ptr(scratch), _ptr(out), M, two_h // 2, K),
+              "tl_hgemm_silu_mul_f16")
+        return out
+
     def prefill_attention(self, q: torch.Tensor, cache_k: torch.Tensor, cache_v: torch.Tensor, start_pos: int):
         """q: [n_heads, S, head_dim] (rotated); caches [max_seq, n_heads, head_dim] holding positions
         < start_pos + S.  Returns [S, n_heads, head_dim]."""

@@ -332,8 +332,8 @@ struct tlm_model {
             ck(tl_hgemm_add_rms_norm_f16(o_c.p, w.wo, x.p, w.ffn_norm, eps, x_residual.p, x_norm.p, S, dim, dim),
                "hgemm_add_rms_norm");
             if (w.w3 == w.w1 + (size_t)hidden * dim && hidden % 8 == 0) {
-                matmul2d(x_norm.p, w.w1, x13.p, S, (size_t)2 * hidden, dim);   // rows of w1.x | w3.x
-                ck(tl_silu_mul_rows_f16(x2.p, x13.p, S, hidden), "silu_mul_rows");
+                // w1.x | w3.x and the gate in the GEMM's epilogue (x13 only where the shape takes two steps)
+                ck(tl_hgemm_silu_mul_f16(x_norm.p, w.w1, x13.p, x2.p, S, hidden, dim), "hgemm_silu_mul");
             } else {
                 matmul2d(x_norm.p, w.w1, x1(S), S, hidden, dim);
                 matmul2d(x_norm.p, w.w3, x3(S), S, hidden, dim);

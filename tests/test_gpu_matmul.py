@@ -369,6 +369,67 @@ def test_hgemm_square_tiles_ragged_edges_and_batches(dev, shape):
     assert torch.equal(Cb.double(), want)
 
 
+GATED_SHAPES = [(128, 11008, 4096), (512, 11008, 4096), (2048, 11008, 4096), (48, 11008, 4096), (16, 11008, 4096),
+                (200, 1000, 4160), (130, 5128, 4096), (700, 6000, 2048), (1, 11008, 4096), (64, 1376, 4100),
+                (300, 72, 128), (3000, 2752, 1024)]
+
+
+@pytest.mark.parametrize("shape", GATED_SHAPES, ids=lambda s: "x".join(map(str, s)))
+def test_hgemm_silu_mul_equals_two_steps(dev, shape):
+    """The two FFN projections with the SwiGLU gate in the GEMM's epilogue against GEMM into a [M, 2*hidden] buffer
+    followed by the gate kernel: the gate sees the same fp16-rounded projections, so every bit agrees.  Shapes: the
+    Llama2-7B w1|w3 at several prompt lengths, hidden not a multiple of any tile, rows past the last tile, K with a tail
+    (two-step path inside the entry), one row (GEMV), a handful of rows (two-step by choice)."""
+    M, hidden, K = shape
+    X = dev.from_numpy(synth.normal_f16(7800 + M, (M, K), 1.0))
+    W13 = dev.from_numpy(synth.normal_f16(7801 + hidden, (2 * hidden, K), 0.02))
+    try:
+        # every workgroup walks all of K from its first tile: both paths then add the same products in the same order
+        dev.lib.tl_set_hgemm_k_rotation(0, 0)
+        dev.lib.tl_set_hgemm_splits(1)
+        want = dev.silu_mul_rows(dev.matmul2d(X, W13))
+        got = dev.hgemm_silu_mul(X, W13)
+        assert got.shape == (M, hidden)
+        assert torch.equal(got, want)
+    finally:
+        dev.lib.tl_set_hgemm_k_rotation(-1, -1)
+        dev.lib.tl_set_hgemm_splits(0)
+    # with the rotated walks of the default dispatch (the order of the fp32 sums then differs from tile to tile):
+    # against float64 of the defining formula, to the tolerance of the GEMM
+    got = dev.hgemm_silu_mul(X, W13)
+    a = X.double() @ W13[:hidden].double().T
+    b = X.double() @ W13[hidden:].double().T
+    ref = (a.half().double() / (1.0 + torch.exp(-a.half().double())) * b.half().double())
+    assert_close_f16(got.cpu().numpy(), ref.cpu().numpy().astype(np.float16), RTOL, 2e-3, f"gated {shape}")
+
+
+def test_hgemm_silu_mul_every_pipelined_variant(dev):
+    """Each pipelined tile shape has a gated build of its own (the pairing of rows follows the wavefront tile): all of
+    them against the two-step path, on a shape with partly filled last tiles in both directions."""
+    M, hidden, K = 300, 1096, 512
+    X = dev.from_numpy(synth.normal_f16(7810, (M, K), 1.0))
+    W13 = dev.from_numpy(synth.normal_f16(7811, (2 * hidden, K), 0.05))
+    names = dev.hgemm_variants()
+    tried = 0
+    try:
+        dev.lib.tl_set_hgemm_k_rotation(0, 0)   # same order of the fp32 sums on both paths
+        dev.lib.tl_set_hgemm_splits(1)
+        want = dev.silu_mul_rows(dev.matmul2d(X, W13))
+        for i, name in enumerate(names):
+            if not name.startswith("p"):
+                continue
+            dev.set_hgemm_variant(i)
+            got = dev.hgemm_silu_mul(X, W13)
+            assert dev.hgemm_last_plan() == (name, 1), name
+            assert torch.equal(got, want), name
+            tried += 1
+    finally:
+        dev.set_hgemm_variant(0)
+        dev.lib.tl_set_hgemm_k_rotation(-1, -1)
+        dev.lib.tl_set_hgemm_splits(0)
+    assert tried >= 10
+
+
 def test_hgemm_k_rotation_and_splits_visit_every_k_tile_once(dev, oracle):
     """Workgroups start their walk over K at a rotated tile and wrap, per split: with small-integer data the
     result is exact whatever the order, so a skipped or repeated K tile shows as a wrong bit."""
