@@ -282,6 +282,15 @@ int tl_prefill_rope_qkv_vt_f16(void* q_out, const void* q, const void* k, const 
                                void* cache_v, const void* rope_table, void* vT, int ldv, int n_tokens, int n_heads,
                                int head_dim);
 
+/* The fused q|k|v projection of a fresh context followed by tl_prefill_rope_qkv_vt_f16: X[n_tokens, K] .
+ * Wqkv[3*n_heads*head_dim, K]^T, then RoPE, cache rows and the transposed values.  When the GEMM splits K (short
+ * prompts), the kernel that rotates reads the fp32 partial sums and adds them itself in split order, so the separate
+ * second pass of the split and one launch are saved; same bits as the two entries called one after the other.
+ * qkv: [n_tokens, 3*n_heads*head_dim] halves, receives the projection when K is not split. */
+int tl_hgemm_prefill_rope_qkv_vt_f16(const void* X, const void* Wqkv, void* qkv, void* q_out, void* cache_k, void* cache_v,
+                                     const void* rope_table, void* vT, int ldv, int n_tokens, int n_heads, int head_dim,
+                                     size_t K);
+
 /* vT[h][d][t] = cache_v[t][h][d] for t < T and 0 for T <= t < ldv (ldv % 8 == 0): the transposed value operand
  * of tl_prefill_attention_f16; the reference builds the same tensor with transpose + contiguous
  * (model/llama2_7b/src/Transformer.cpp:66-80). */

@@ -89,6 +89,7 @@ _PROTOS = {
     "tl_gemv_silu_mul_f16": (_i, [_vp, _vp, _vp, _sz, _sz]),
     "tl_prefill_rope_qkv_f16": (_i, [_vp, _vp, _vp, _vp, _sz, _vp, _vp, _vp, _i, _i, _i, _i]),
     "tl_prefill_rope_qkv_vt_f16": (_i, [_vp, _vp, _vp, _vp, _sz, _vp, _vp, _vp, _vp, _i, _i, _i, _i]),
+    "tl_hgemm_prefill_rope_qkv_vt_f16": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _sz]),
     "tl_scaled_causal_softmax_f16": (_i, [_vp, _u16, _i, _i, _i]),
     "tl_silu_mul_rows_f16": (_i, [_vp, _vp, _sz, _sz]),
     "tl_gather_vt_f16": (_i, [_vp, _vp, _i, _i, _i, _i]),

@@ -381,14 +381,36 @@ prefill_rope_qkv_kernel(half_t* q_out, const half_t* q, const half_t* k, const h
 // prefill_rope_qkv_kernel and gather_vt_kernel in one pass for a fresh context (start_pos 0, so the new tokens are
 // all there is to transpose): workgroup (64-token tile, head), 16-byte accesses throughout; the tile of v goes
 // through LDS and leaves transposed, 128 contiguous bytes per head_dim row, zero beyond the last token.
-template <int D>
+// SLABS: the projection's K was split and its fp32 partial sums [splits][n_tokens][ld] have not been added up yet; q, k
+// and v then only carry the column where their section starts (the column number times two as the pointer's value) and every value read is
+// half(partial[0] + partial[1] + ...), the sum and rounding of splitk_reduce_kernel.
+template <int D, bool SLABS>
 __global__ void __launch_bounds__(256)
 prefill_rope_qkv_vt_kernel(half_t* q_out, const half_t* q, const half_t* k, const half_t* v, size_t ld, half_t* cache_k,
-                           half_t* cache_v, const half_t* rope_table, half_t* vT, int ldv, int n_tokens, int n_heads) {
+                           half_t* cache_v, const half_t* rope_table, half_t* vT, int ldv, int n_tokens, int n_heads,
+                           const float* slabs, int splits, size_t slab_elems) {
+    auto load8 = [&](const half_t* base, size_t off) -> half8_t {
+        if constexpr (SLABS) {
+            const float* p = slabs + reinterpret_cast<uintptr_t>(base) / sizeof(half_t) + off;   // base: a column, not an address
+            float4_t lo = *reinterpret_cast<const float4_t*>(p), hi = *reinterpret_cast<const float4_t*>(p + 4);
+            for (int sp = 1; sp < splits; ++sp) {
+                lo += *reinterpret_cast<const float4_t*>(p + (size_t)sp * slab_elems);
+                hi += *reinterpret_cast<const float4_t*>(p + (size_t)sp * slab_elems + 4);
+            }
+            const half8_t r = {(half_t)lo[0], (half_t)lo[1], (half_t)lo[2], (half_t)lo[3],
+                               (half_t)hi[0], (half_t)hi[1], (half_t)hi[2], (half_t)hi[3]};
+            return r;
+        } else {
+            return *reinterpret_cast<const half8_t*>(base + off);
+        }
+    };
     constexpr int CH = D / 8;                     // 16-byte chunks per head row
     __shared__ __attribute__((aligned(16))) half_t vt_tile[64][D + 8];
     const int h = blockIdx.y;
     const int s0 = blockIdx.x * 64;
+    // a grid three deep gives q, k and v a workgroup each (short prompts: three times the workgroups pull on the slabs)
+    const bool do_q = gridDim.z == 1 || blockIdx.z == 0, do_k = gridDim.z == 1 || blockIdx.z == 1,
+               do_v = gridDim.z == 1 || blockIdx.z == 2;
     const half8_t zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
     for (int it = threadIdx.x; it < 64 * CH; it += 256) {
         const int sl = it / CH, c = it % CH;
@@ -396,17 +418,20 @@ prefill_rope_qkv_vt_kernel(half_t* q_out, const half_t* q, const half_t* k, cons
         half8_t vv = zero8;
         if (s < n_tokens) {
             const size_t in_off = (size_t)s * ld + (size_t)h * D + c * 8;
-            const half8_t cs = *reinterpret_cast<const half8_t*>(rope_table + ((size_t)s * (D / 2) + c * 4) * 2);
-            const half8_t qr = rope_chunk_cs(*reinterpret_cast<const half8_t*>(q + in_off), cs);
-            const half8_t kr = rope_chunk_cs(*reinterpret_cast<const half8_t*>(k + in_off), cs);
-            vv = *reinterpret_cast<const half8_t*>(v + in_off);
-            *reinterpret_cast<half8_t*>(q_out + ((size_t)h * n_tokens + s) * D + c * 8) = qr;
             const size_t c_off = ((size_t)s * n_heads + h) * D + c * 8;
-            *reinterpret_cast<half8_t*>(cache_k + c_off) = kr;
-            *reinterpret_cast<half8_t*>(cache_v + c_off) = vv;
+            half8_t cs = zero8;
+            if (do_q || do_k) cs = *reinterpret_cast<const half8_t*>(rope_table + ((size_t)s * (D / 2) + c * 4) * 2);
+            if (do_q)
+                *reinterpret_cast<half8_t*>(q_out + ((size_t)h * n_tokens + s) * D + c * 8) = rope_chunk_cs(load8(q, in_off), cs);
+            if (do_k) *reinterpret_cast<half8_t*>(cache_k + c_off) = rope_chunk_cs(load8(k, in_off), cs);
+            if (do_v) {
+                vv = load8(v, in_off);
+                *reinterpret_cast<half8_t*>(cache_v + c_off) = vv;
+            }
         }
-        *reinterpret_cast<half8_t*>(&vt_tile[sl][c * 8]) = vv;
+        if (do_v) *reinterpret_cast<half8_t*>(&vt_tile[sl][c * 8]) = vv;
     }
+    if (!do_v) return;
     __syncthreads();
     for (int it = threadIdx.x; it < D * 8; it += 256) {
         const int d = it / 8, j = it % 8;
@@ -1120,11 +1145,50 @@ int tl_prefill_rope_qkv_vt_f16(void* q_out, const void* q, const void* k, const 
     auto launch = [&](auto kernel) {
         hipLaunchKernelGGL(kernel, grid, dim3(256), 0, tl::stream(), (tl::half_t*)q_out, (const tl::half_t*)q,
                            (const tl::half_t*)k, (const tl::half_t*)v, row_stride, (tl::half_t*)cache_k, (tl::half_t*)cache_v,
-                           (const tl::half_t*)rope_table, (tl::half_t*)vT, ldv, n_tokens, n_heads);
+                           (const tl::half_t*)rope_table, (tl::half_t*)vT, ldv, n_tokens, n_heads, (const float*)nullptr, 1,
+                           (size_t)0);
     };
-    if (head_dim == 64) launch(tl::prefill_rope_qkv_vt_kernel<64>);
-    else launch(tl::prefill_rope_qkv_vt_kernel<128>);
+    if (head_dim == 64) launch(tl::prefill_rope_qkv_vt_kernel<64, false>);
+    else launch(tl::prefill_rope_qkv_vt_kernel<128, false>);
     TL_CHECK_LAUNCH("prefill_rope_qkv_vt_kernel");
+    return TL_OK;
+}
+
+int tl_hgemm_prefill_rope_qkv_vt_f16(const void* X, const void* Wqkv, void* qkv, void* q_out, void* cache_k, void* cache_v,
+                                     const void* rope_table, void* vT, int ldv, int n_tokens, int n_heads, int head_dim,
+                                     size_t K) {
+    TL_ENSURE_INIT();
+    TL_REQUIRE(X && Wqkv && qkv, "tl_hgemm_prefill_rope_qkv_vt_f16: null pointer");
+    TL_REQUIRE(n_tokens >= 1 && n_heads >= 1 && (head_dim == 64 || head_dim == 128),
+               "tl_hgemm_prefill_rope_qkv_vt_f16: bad sizes");
+    const size_t dim = (size_t)n_heads * head_dim, N = 3 * dim, M = (size_t)n_tokens;
+    float* slabs = nullptr;
+    int splits = 1;
+    tl::Workspace::Lease lease;   // keeps the split-K slabs in place until the kernel that reads them is enqueued
+    int rc = M == 1 ? tl::launch_gemv(X, Wqkv, qkv, N, K, 1, 0, 0, 0, 0)
+                    : tl::launch_hgemm(X, Wqkv, qkv, M, N, K, 1, 0, 0, 0, &slabs, &splits, &lease);
+    if (rc != TL_OK) return rc;
+    const tl::half_t* base = (const tl::half_t*)qkv;
+    if (splits <= 1)
+        return tl_prefill_rope_qkv_vt_f16(q_out, base, base + dim, base + 2 * dim, N, cache_k, cache_v, rope_table, vT, ldv,
+                                          n_tokens, n_heads, head_dim);
+    // same argument checks as the entry above, the projections read from the slabs
+    TL_REQUIRE(q_out && cache_k && cache_v && rope_table && vT, "tl_hgemm_prefill_rope_qkv_vt_f16: null pointer");
+    TL_REQUIRE(n_heads <= 65535 && ldv % 64 == 0 && ldv >= n_tokens,
+               "tl_hgemm_prefill_rope_qkv_vt_f16: ldv=%d must be a multiple of 64 that covers the tokens", ldv);
+    TL_REQUIRE(tl::aligned16(q_out) && tl::aligned16(cache_k) && tl::aligned16(cache_v) && tl::aligned16(rope_table) &&
+                   tl::aligned16(vT) && tl::aligned16(slabs),
+               "tl_hgemm_prefill_rope_qkv_vt_f16: pointers must be 16-byte aligned");
+    dim3 grid((unsigned)(ldv / 64), (unsigned)n_heads, 3);
+    auto column = [](size_t col) { return reinterpret_cast<const tl::half_t*>((uintptr_t)(col * sizeof(tl::half_t))); };
+    auto launch = [&](auto kernel) {
+        hipLaunchKernelGGL(kernel, grid, dim3(256), 0, tl::stream(), (tl::half_t*)q_out, column(0), column(dim),
+                           column(2 * dim), N, (tl::half_t*)cache_k, (tl::half_t*)cache_v, (const tl::half_t*)rope_table,
+                           (tl::half_t*)vT, ldv, n_tokens, n_heads, (const float*)slabs, splits, M * N);
+    };
+    if (head_dim == 64) launch(tl::prefill_rope_qkv_vt_kernel<64, true>);
+    else launch(tl::prefill_rope_qkv_vt_kernel<128, true>);
+    TL_CHECK_LAUNCH("prefill_rope_qkv_vt_kernel<slabs>");
     return TL_OK;
 }
 

@@ -419,6 +419,26 @@ class HipDevice:
                                                   _ptr(cache_v), _ptr(table), _ptr(vT), ldv, S, n_heads, D),
               "tl_prefill_rope_qkv_vt_f16")
         return out, vT
+
+    def hgemm_prefill_rope_qkv_vt(self, X: torch.Tensor, Wqkv: torch.Tensor, cache_k: torch.Tensor, cache_v: torch.Tensor,
+                                  table: torch.Tensor, n_heads: int):
+        """The fused q|k|v projection of a fresh context and prefill_rope_qkv_vt in one call (the rotating kernel adds
+        up a split K itself).  X [S, K], Wqkv [3*dim, K].  Returns (q [n_heads, S, D], vT [n_heads, D, ldv])."""
+        _req(X, name="X"), _req(Wqkv, name="Wqkv")
+        S, K = X.shape
+        N, K2 = Wqkv.shape
+        if K != K2 or N % (3 * n_heads):
+            raise ValueError("Shape mismatch: X [S, K] against Wqkv [3*n_heads*head_dim, K]")
+        D = N // 3 // n_heads
+        ldv = (S + 63) // 64 * 64
+        qkv = torch.empty((S, N), dtype=torch.float16, device=X.device)
+        out = torch.empty((n_heads, S, D), dtype=torch.float16, device=X.device)
+        vT = torch.empty((n_heads, D, ldv), dtype=torch.float16, device=X.device)
+        check(self.lib.tl_hgemm_prefill_rope_qkv_vt_f16(_ptr(X), _ptr(Wqkv), _ptr(qkv), _ptr(out), _ptr(cache_k), _ptr(cache_v),
+                                                        _ptr(table), _ptr(vT), ldv, S, n_heads, D, K),
+              "tl_hgemm_prefill_rope_qkv_vt_f16")
+        return out, vT
+
     def scaled_causal_softmax(self, scores: torch.Tensor, divisor: float, start_pos: int) -> torch.Tensor:
         """In place on scores [n_heads, S, start_pos + S]: divide by half(divisor), causal mask, softmax."""
         _req(scores, name="scores")

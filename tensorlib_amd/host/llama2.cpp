@@ -291,7 +291,15 @@ struct tlm_model {
             const size_t dd = (size_t)dim * dim;
             const half *q, *k, *v;
             size_t ld;
-            if (w.wk == w.wq + dd && w.wv == w.wk + dd) {
+            const int ldv = (T + 63) / 64 * 64;
+            bool projected_and_rotated = false;
+            if (w.wk == w.wq + dd && w.wv == w.wk + dd && (D == 64 || D == 128) && start_pos == 0) {
+                // q | k | v in one GEMM, rotated and scattered by the kernel that also adds up a split K
+                ck(tl_hgemm_prefill_rope_qkv_vt_f16(x_norm.p, w.wq, qkv.p, xq_c.p, cache_k[l].p, cache_v[l].p, rope_table.p,
+                                                    values_c.p, ldv, S, H, D, dim), "hgemm_prefill_rope_qkv_vt");
+                projected_and_rotated = true;
+                q = k = v = nullptr; ld = 0;
+            } else if (w.wk == w.wq + dd && w.wv == w.wk + dd) {
                 matmul2d(x_norm.p, w.wq, qkv.p, S, (size_t)3 * dim, dim);   // rows of q | k | v
                 q = qkv.p; k = qkv.p + dim; v = qkv.p + 2 * dim; ld = (size_t)3 * dim;
             } else {
@@ -300,9 +308,10 @@ struct tlm_model {
                 matmul2d(x_norm.p, w.wv, xv(S), S, dim, dim);
                 q = xq(S); k = xk(S); v = xv(S); ld = dim;
             }
-            const int ldv = (T + 63) / 64 * 64;
-            const bool one_pass = (D == 64 || D == 128) && start_pos == 0 && ld % 8 == 0;
-            if (one_pass) {
+            const bool one_pass = projected_and_rotated || ((D == 64 || D == 128) && start_pos == 0 && ld % 8 == 0);
+            if (projected_and_rotated) {
+                // nothing left to do before the attention
+            } else if (one_pass) {
                 // a fresh context: the transposed values are written along with the rotated q, k and the cache rows
                 ck(tl_prefill_rope_qkv_vt_f16(xq_c.p, q, k, v, ld, cache_k[l].p, cache_v[l].p, rope_table.p, values_c.p, ldv,
                                               S, H, D), "prefill_rope_qkv_vt");

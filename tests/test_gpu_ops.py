@@ -361,6 +361,25 @@ def test_rope_table_bits_equal_the_cpu_loop(dev, oracle, D):
     assert differs.shape == (2048, D // 2) and not differs[0].any()
 
 
+@pytest.mark.parametrize("S,H,D,K", [(128, 32, 128, 4096), (64, 32, 128, 4096), (100, 32, 128, 4096), (512, 32, 128, 4096),
+                                     (2, 32, 128, 4096), (1, 8, 64, 512), (40, 8, 64, 8192), (300, 4, 128, 1024)])
+def test_hgemm_prefill_rope_qkv_vt_equals_separate_calls(dev, S, H, D, K):
+    """Projection + rotation in one call against tl_matmul2d_f16 followed by tl_prefill_rope_qkv_vt_f16: rotated q, both
+    cache rows and the transposed values bit for bit, at prompt lengths where the GEMM splits K (the rotating kernel then
+    reads the fp32 partial sums) and where it does not."""
+    dim = H * D
+    X = dev.from_numpy(synth.normal_f16(170 + S, (S, K), 1.0))
+    W = dev.from_numpy(synth.normal_f16(171 + S, (3 * dim, K), 0.02))
+    table = dev.rope_table(max(S, 8), D)
+    qkv = dev.matmul2d(X, W)
+    k1, v1 = dev.empty(S, H, D), dev.empty(S, H, D)
+    q1, vT1 = dev.prefill_rope_qkv_vt(qkv[:, :dim], qkv[:, dim:2 * dim], qkv[:, 2 * dim:], k1, v1, table, H)
+    split = dev.hgemm_last_plan()[1]
+    k2, v2 = dev.empty(S, H, D), dev.empty(S, H, D)
+    q2, vT2 = dev.hgemm_prefill_rope_qkv_vt(X, W, k2, v2, table, H)
+    assert torch.equal(q2, q1) and torch.equal(k2, k1) and torch.equal(v2, v1) and torch.equal(vT2, vT1), f"splits {split}"
+
+
 @pytest.mark.parametrize("D", [64, 128])
 @pytest.mark.parametrize("chunk", [64, 128, 256])
 def test_decode_attention_every_chunk_size_vs_chain(dev, oracle, chunk, D):
