@@ -403,6 +403,30 @@ def test_hgemm_silu_mul_equals_two_steps(dev, shape):
     assert_close_f16(got.cpu().numpy(), ref.cpu().numpy().astype(np.float16), RTOL, 2e-3, f"gated {shape}")
 
 
+def test_hgemm_silu_mul_drawn_shapes(dev):
+    """Forty drawn shapes (rows 2..700, hidden a multiple of 8 up to 3000, K a multiple of 64 up to 2048) through the
+    automatic dispatch: tiles partly filled in both directions, column ranges, every tile shape the dispatch reaches."""
+    rng = np.random.default_rng(20240611)
+    seen = set()
+    try:
+        dev.lib.tl_set_hgemm_k_rotation(0, 0)
+        dev.lib.tl_set_hgemm_splits(1)
+        for i in range(40):
+            M = int(rng.integers(2, 701))
+            hidden = 8 * int(rng.integers(1, 376))
+            K = 64 * int(rng.integers(1, 33))
+            X = dev.from_numpy(synth.normal_f16(7900 + i, (M, K), 1.0))
+            W13 = dev.from_numpy(synth.normal_f16(8000 + i, (2 * hidden, K), 0.05))
+            want = dev.silu_mul_rows(dev.matmul2d(X, W13))
+            got = dev.hgemm_silu_mul(X, W13)
+            seen.add(dev.hgemm_last_plan()[0])
+            assert torch.equal(got, want), (M, hidden, K, dev.hgemm_last_plan())
+    finally:
+        dev.lib.tl_set_hgemm_k_rotation(-1, -1)
+        dev.lib.tl_set_hgemm_splits(0)
+    assert len(seen) >= 2, seen
+
+
 def test_hgemm_silu_mul_every_pipelined_variant(dev):
     """Each pipelined tile shape has a gated build of its own (the pairing of rows follows the wavefront tile): all of
     them against the two-step path, on a shape with partly filled last tiles in both directions."""
