@@ -819,7 +819,7 @@ static HgemmPlan plan_many_rows(size_t M, size_t N, size_t K, int cus, bool can_
 // column range of C and the remaining columns as a second launch with whatever tiles suit THAT problem
 // (launch_hgemm; 2048x11008x4096: 344 big tiles = one round + 88 tiles, or one round + 176 tiles of 128x256).
 // Up to 512 rows and from 5120 columns on, 128x128 tiles on four wavefronts, split over K until they fill one round
-// of the chip, are as fast as or faster than the rules of pick_variant wherever they fill at least 70 % of the
+// of the chip, are as fast as or faster than the rules of pick_variant wherever they fill at least 67 % of the
 // compute units (60 % from 192 rows on) with K loops of 1024 to 8192 (sweep of seven tile shapes x six split counts
 // over 152 shapes, M = 48 .. 512, projections of Llama-size models 2048 to 8192 wide: 256x8192x8192 71.6 -> 52.8 us,
 // 384x6144x4096 52.1 -> 37.7, 256x5120x5120 38.0 -> 29.7, 48x12288x4096 26.8 -> 23.9; at most 5 % slower on the shapes
@@ -841,7 +841,7 @@ static int square_tile_splits(size_t M, size_t N, size_t K, int cus, bool can_sp
         sp = s;
         if ((double)((KT + s - 1) / s) * per_k_us <= hbm_us) break;
     }
-    if (K > (size_t)sp * 8192 || t * sp * 10 < (size_t)cus * (M >= 192 ? 6 : 7)) return 0;
+    if (K > (size_t)sp * 8192 || t * sp * 100 < (size_t)cus * (M >= 192 ? 60 : 67)) return 0;
     return sp;
 }
 
