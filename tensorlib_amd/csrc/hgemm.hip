@@ -860,7 +860,10 @@ static int pick_variant(size_t M, size_t N, size_t K, int cus, bool can_split) {
         // (not with a very long K that two splits of 128x256 tiles cover in one round: 512x8192x28672 319 -> 237 us)
         const bool split_wide = can_split && K >= 16384 && M >= 256 && tiles(128, 256) * 2 <= (size_t)cus;
         if (M > 128 && tiles(128, 192) >= enough && tiles(128, 192) <= (size_t)cus && !split_wide) return v_few_128x192;
-        if (M > 128 && tiles(128, 256) >= enough) return v_mid;   // measured ahead of 256x128 at equal tile counts
+        // one row of 256-row tiles reads every row of W once; two rows of 128-row tiles read it twice (38 shapes with
+        // 192 and 256 rows: 256x128 ahead of 128x256 by 1-9 %, 256x32000x4096 90.4 -> 82.3 us)
+        if (M > 128 && M <= 256 && tiles(256, 128) >= enough) return v_few_256x128;
+        if (M > 128 && tiles(128, 256) >= enough) return v_mid;   // from 257 rows on ahead of 256x128 at equal tile counts
         if (M > 128 && tiles(256, 128) >= enough) return v_few_256x128;
         // A long K is split instead of narrowing the tile: wider tiles pull fewer bytes through a CU per output, and
         // the slabs are small next to W (256x4096x11008: 128x128 tiles on four splits 40-43 us, 128x64 on two 48-49 us;
