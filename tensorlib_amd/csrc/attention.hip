@@ -22,7 +22,7 @@ namespace tl {
 // 0: automatic, 1: one wavefront per 32 query rows, 2: LDS-tiled workgroups of 128 query rows (tuning hook)
 static std::atomic<int> g_prefill_attention_variant{0};
 // where the chunk partials of a head are merged: 0 = automatic, 1 = by the workgroup that finishes the head's last
-// chunk, 2 = by a second launch
+// chunk, 2 = by a second launch, 3 = like 1 with a release/acquire ticket and plain accesses to the partials
 static std::atomic<int> g_decode_merge_mode{0};
 // Up to this many chunks the in-kernel merge is ahead (384 positions: 7.6 against 10.2 us for the pair of launches;
 // 1024 positions: equal; 1951 positions: 14.7 against 13.2 us, the merging workgroup's serial walk over 31 partials
@@ -143,7 +143,7 @@ template <int LPR, int ROPE, int CHUNK>
 __global__ void __launch_bounds__(kAttnThreads)
 decode_attn_partial_kernel(half_t* out, float* partial, const half_t* q, half_t* cache_k,
                            half_t* cache_v, const half_t* rope_table, int T, int n_heads, float inv_scale,
-                           int n_chunks, unsigned* tickets) {
+                           int n_chunks, unsigned* tickets, int ordered) {
     constexpr int D = LPR * 8;
     constexpr int GROUPS = kAttnThreads / LPR;
     static_assert(CHUNK % 64 == 0 && CHUNK <= kAttnThreads && CHUNK % (kAttnThreads / LPR) == 0, "chunk size");
@@ -293,7 +293,7 @@ decode_attn_partial_kernel(half_t* out, float* partial, const half_t* q, half_t*
             out[(size_t)h * D + tid] = (half_t)(o / l);
         } else {
             float* p = partial + ((size_t)h * n_chunks + chunk) * (D + 2);
-            if (tickets) {
+            if (tickets && !ordered) {
                 // device-coherent stores: the workgroup that merges may sit on another XCD, behind another L2
                 __hip_atomic_store(p + 2 + tid, o, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                 if (tid == 0) {
@@ -307,21 +307,32 @@ decode_attn_partial_kernel(half_t* out, float* partial, const half_t* q, half_t*
         }
     }
     if (tickets == nullptr || n_chunks == 1) return;
-    // One launch instead of two: the workgroup that finishes a head's last chunk merges the head.  Its partials
-    // have been acknowledged (vmcnt(0)) before its ticket is drawn, tickets and partials are device-coherent
-    // accesses, and the merge walks the chunks in index order, so the result has the bits of the two-launch path.
+    // One launch instead of two: the workgroup that finishes a head's last chunk merges the head, walking the chunks
+    // in index order, so the result has the bits of the two-launch path.
+    // What orders the partials before the merge (ordered == 0, the default): the partials leave as device-coherent
+    // stores (write-through, sc1), every wavefront waits until its stores are acknowledged (s_waitcnt vmcnt(0):
+    // on this ISA a store counts as done when the coherent level holds it), the workgroup barrier collects those
+    // waits, and only then is the ticket drawn; the workgroup that draws the last ticket reads the partials with
+    // device-coherent loads issued after the ticket's value has returned.  That is an ordering by instruction
+    // completion, which the HIP memory model does not spell out for relaxed atomics.  ordered == 1 is the same
+    // protocol in the model's own terms: plain stores, a release/acquire read-modify-write at device scope on the
+    // ticket, plain loads.  It costs a write-back of this XCD's L2 per workgroup and an invalidate in the merging
+    // one (measured: slower, see tl_set_decode_attention_merge), so it is kept as the tested alternative, not the
+    // default.
     __shared__ int s_last;
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    if (!ordered) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
     if (tid == 0) {
-        const unsigned t = __hip_atomic_fetch_add(tickets + h, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        const unsigned t = ordered ? __hip_atomic_fetch_add(tickets + h, 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT)
+                                   : __hip_atomic_fetch_add(tickets + h, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         const int last = (t + 1u == (unsigned)n_chunks);
         if (last) __hip_atomic_store(tickets + h, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // ready for the next call
         s_last = last;
     }
     __syncthreads();
     if (!s_last || tid >= D) return;
-    merge_head<true>(out, partial + (size_t)h * n_chunks * (D + 2), h, D, n_chunks, tid);
+    if (ordered) merge_head<false>(out, partial + (size_t)h * n_chunks * (D + 2), h, D, n_chunks, tid);
+    else merge_head<true>(out, partial + (size_t)h * n_chunks * (D + 2), h, D, n_chunks, tid);
 }
 
 // Second pass for long contexts: merge the chunk partials of one head.  (Short contexts merge inside the first
@@ -981,6 +992,16 @@ int attention_static_scratch(float** out) {
     return TL_OK;
 }
 
+// Puts the ticket words of both scratch buffers back to zero (after a launch that did not complete).
+int attention_reset_tickets() {
+    int rc = g_partials.zero_head(kAttnTicketWords);
+    if (rc != TL_OK) return rc;
+    float* st = nullptr;
+    rc = attention_static_scratch(&st);
+    if (rc != TL_OK) return rc;
+    return launch_fill_f16(st, 0, kAttnTicketWords * 2);
+}
+
 }  // namespace tl
 
 extern "C" {
@@ -1004,8 +1025,9 @@ static int launch_decode_attention(void* out, const void* q, void* cache_k, void
     const int n_chunks = (T + chunk - 1) / chunk;
     TL_REQUIRE(n_chunks <= 65535, "%s: T=%d too long", name, T);
     tl::Workspace::Lease lease;   // held until both kernels are enqueued
-    // [one ticket per head, padded to 64 words][partials]; tickets are zero between calls
-    const size_t ticket_words = ((size_t)n_heads + 63) / 64 * 64;
+    // [kAttnTicketWords ticket words, one per head][partials]; tickets are zero between calls.  The ticket region has
+    // one size for every call, so partials of one call never land where another call keeps tickets.
+    const size_t ticket_words = tl::kAttnTicketWords;
     const size_t ws_floats = ticket_words + (size_t)n_heads * n_chunks * (head_dim + 2);
     float* ws = static_ws;
     if (static_ws) {
@@ -1019,7 +1041,9 @@ static int launch_decode_attention(void* out, const void* q, void* cache_k, void
         ws = lease.ptr;
     }
     const int merge_mode = tl::g_decode_merge_mode.load();
-    const bool in_kernel = merge_mode == 1 || (merge_mode == 0 && n_chunks <= tl::kMergeInKernelMaxChunks);
+    // more heads than ticket words: the second kernel merges
+    const bool in_kernel = (size_t)n_heads <= ticket_words &&
+                           (merge_mode == 1 || merge_mode == 3 || (merge_mode == 0 && n_chunks <= tl::kMergeInKernelMaxChunks));
     unsigned* tickets = (ws && in_kernel) ? reinterpret_cast<unsigned*>(ws) : nullptr;
     float* partials = ws ? ws + ticket_words : nullptr;
     // the reference divides the scores by half(sqrt(head_dim)) (Transformer.cpp:94)
@@ -1030,7 +1054,7 @@ static int launch_decode_attention(void* out, const void* q, void* cache_k, void
     auto launch = [&](auto kernel) {
         hipLaunchKernelGGL(kernel, grid, dim3(tl::kAttnThreads), 0, st, (tl::half_t*)out, partials,
                            (const tl::half_t*)q, (tl::half_t*)cache_k, (tl::half_t*)cache_v,
-                           (const tl::half_t*)rope_table, T, n_heads, inv_scale, n_chunks, tickets);
+                           (const tl::half_t*)rope_table, T, n_heads, inv_scale, n_chunks, tickets, merge_mode == 3 ? 1 : 0);
     };
     const int rope = fuse_rope ? (rope_table ? 1 : 2) : 0;
     auto launch_chunk = [&](auto lpr, auto rp) {
@@ -1257,7 +1281,7 @@ int tl_prefill_attention_f16(void* out, const void* q, const void* cache_k, cons
 }
 
 int tl_set_decode_attention_merge(int mode) {
-    TL_REQUIRE(mode >= 0 && mode <= 2, "tl_set_decode_attention_merge: %d out of range [0,2]", mode);
+    TL_REQUIRE(mode >= 0 && mode <= 3, "tl_set_decode_attention_merge: %d out of range [0,3]", mode);
     tl::g_decode_merge_mode = mode;
     return TL_OK;
 }

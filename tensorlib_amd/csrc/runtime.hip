@@ -63,10 +63,12 @@ int ensure_init() {
     return init_locked(dev);
 }
 
+static std::atomic<bool> g_ws_in_use{false};
+bool workspaces_in_use() { return g_ws_in_use.load(std::memory_order_acquire); }
+
 int Workspace::acquire(size_t floats, size_t min_floats, const char* what, Lease* lease) {
     lease->lock = std::unique_lock<std::mutex>(mu_);
     hipStream_t st = stream();
-    if (used_ && st != last_stream_) TL_HIP_TRY(hipStreamSynchronize(last_stream_));
     if (floats > floats_) {
         if (ptr_) {
             TL_HIP_TRY(hipStreamSynchronize(st));
@@ -82,13 +84,19 @@ int Workspace::acquire(size_t floats, size_t min_floats, const char* what, Lease
                              hipGetErrorString(e));
         }
         floats_ = want;
-        // users keep counters in the buffer that are zero between calls (attention tickets): start from zeros
-        TL_HIP_TRY(hipMemsetAsync(ptr_, 0, want * sizeof(float), st));
+        // users keep counters in the buffer that are zero between calls (tickets): start from zeros
+        int rc = launch_fill_f16(ptr_, 0, want * 2);
+        if (rc != TL_OK) return rc;
     }
-    last_stream_ = st;
-    used_ = true;
+    g_ws_in_use.store(true, std::memory_order_release);
     lease->ptr = ptr_;
     return TL_OK;
+}
+
+int Workspace::zero_head(size_t floats) {
+    std::lock_guard<std::mutex> lk(mu_);
+    if (!ptr_) return TL_OK;
+    return launch_fill_f16(ptr_, 0, (floats < floats_ ? floats : floats_) * 2);
 }
 
 }  // namespace tl
@@ -108,7 +116,11 @@ const char* tl_version(void) { return "tensorlib_amd 0.1 gfx950"; }
 int tl_device_cu_count(void) { return tl::g_ready.load(std::memory_order_acquire) ? tl::g_info.cu_count : 0; }
 
 int tl_set_stream(void* hip_stream) {
-    tl::g_stream = static_cast<hipStream_t>(hip_stream);
+    hipStream_t next = static_cast<hipStream_t>(hip_stream);
+    // Work queued on the stream being replaced may still use the library's scratch buffers, which the next call on
+    // the new stream reuses: drain it here, while the caller's handle is certainly still valid.
+    if (next != tl::g_stream && tl::g_ws_in_use.exchange(false)) TL_HIP_TRY(hipStreamSynchronize(tl::g_stream));
+    tl::g_stream = next;
     return TL_OK;
 }
 void* tl_get_stream(void) { return tl::g_stream; }
@@ -162,6 +174,13 @@ int tl_synchronize(void) {
     TL_ENSURE_INIT();
     TL_HIP_TRY(hipStreamSynchronize(tl::stream()));
     return TL_OK;
+}
+
+int tl_reset_scratch(void) {
+    TL_ENSURE_INIT();
+    int rc = tl::attention_reset_tickets();
+    if (rc != TL_OK) return rc;
+    return tl::splitk_reset_tickets();
 }
 
 }  // extern "C"

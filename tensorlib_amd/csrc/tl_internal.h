@@ -41,8 +41,10 @@ int ensure_init();
 // Library-owned fp32 device scratch that grows on demand (split-K partial sums, attention chunk partials).
 // acquire() returns with the buffer's mutex held by the lease: the caller keeps the lease alive until every
 // kernel that touches the pointer is enqueued, so no other host thread can grow (free) the buffer in between.
-// Reuse is ordered by the stream: when the library's stream changed since the last user, that stream is drained
-// first.
+// Reuse is ordered by the library's stream; tl_set_stream drains the stream it replaces once a workspace has been
+// used on it, so no stream handle outlives its owner here.  A buffer starts out all zero (written by a fill kernel,
+// which a stream capture can record) and its first `head` floats hold the users' counters, which every kernel
+// leaves at zero when it completes; zero_head() puts them back after a launch that did not.
 class Workspace {
  public:
     struct Lease {
@@ -50,14 +52,23 @@ class Workspace {
         float* ptr = nullptr;
     };
     int acquire(size_t floats, size_t min_floats, const char* what, Lease* lease);
+    int zero_head(size_t floats);
 
  private:
     std::mutex mu_;
     float* ptr_ = nullptr;
     size_t floats_ = 0;
-    hipStream_t last_stream_ = nullptr;
-    bool used_ = false;
 };
+// true once any workspace has been handed out since the library's stream was last drained by tl_set_stream
+bool workspaces_in_use();
+
+// Counter words at the head of the scratch buffers.  Decode attention: one ticket per head (launches with more
+// heads merge with a second kernel).  Split-K GEMM: one ticket per C tile (launches with more tiles reduce with a
+// second kernel).
+constexpr size_t kAttnTicketWords = 1024;
+constexpr size_t kSplitkTicketWords = 4096;
+int attention_reset_tickets();   // zero the ticket words of both attention scratch buffers (workspace and static)
+int splitk_reset_tickets();
 
 // Looks up (once per device) the device address of the static scratch array behind
 // tl_decode_attention_rope_static_f16 for the current device; `out` may be null.

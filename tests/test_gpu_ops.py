@@ -424,6 +424,44 @@ def test_decode_attention_merge_inside_the_launch_equals_second_launch(dev, T):
         dev.lib.tl_set_decode_attention_merge(0)
 
 
+def test_decode_attention_ticket_region_does_not_move_with_the_head_count(dev):
+    """A call with few heads and several chunks leaves partial results in the scratch buffer; a later call with more
+    heads must not find them where it keeps its tickets.  32 heads then 96 heads at 300 positions, through the entry
+    with the grown-on-demand workspace and the one with the static array, against the second-launch merge; and the
+    release/acquire form of the in-launch merge gives the same bits."""
+    D, T = 128, 300
+    for static in (False, True):
+        for H in (32, 96, 32, 96):
+            qkv = dev.from_numpy(synth.normal_f16(170 + H, (3, H, D), 1.0))
+            ck0 = synth.normal_f16(171 + H, (T, H, D), 1.0)
+            cv0 = synth.normal_f16(172 + H, (T, H, D), 1.0)
+            table = dev.rope_table(T, D)
+            outs = {}
+            try:
+                for mode in (2, 1, 3, 0):
+                    dev.lib.tl_set_decode_attention_merge(mode)
+                    ck, cv = dev.from_numpy(ck0), dev.from_numpy(cv0)
+                    out = dev.empty(H, D)
+                    dev.decode_attention_rope(qkv, ck, cv, T - 1, table, out=out, static_scratch=static)
+                    outs[mode] = out.clone()
+            finally:
+                dev.lib.tl_set_decode_attention_merge(0)
+            for mode in (1, 3, 0):
+                assert torch.equal(outs[mode], outs[2]), (static, H, mode)
+
+
+def test_decode_attention_more_heads_than_tickets_merges_with_the_second_kernel(dev, oracle):
+    """More heads than the scratch buffer has ticket words: the launch takes the second-kernel merge by itself."""
+    H, D, T = 1040, 64, 130
+    q = synth.normal_f16(180, (H, D), 1.0)
+    ck = synth.normal_f16(181, (T, H, D), 1.0)
+    cv = synth.normal_f16(182, (T, H, D), 1.0)
+    got = dev.decode_attention(dev.from_numpy(q), dev.from_numpy(ck), dev.from_numpy(cv), T).cpu().numpy()
+    rows = [0, 63, 64, 1023, 1024, 1039]
+    want = _attention_chain_oracle(oracle, q[rows], ck[:, rows], cv[:, rows], T)
+    assert_close_f16(got[rows], want, RTOL, ATOL, "1040 heads")
+
+
 def test_decode_attention_repeated_calls_reuse_counters(dev, oracle):
     """Many calls in a row with different numbers of chunks share one partials workspace: all of
     them have to agree with the CPU chain."""
