@@ -54,7 +54,15 @@ def parse_args():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", choices=["gemv", "hgemm", "decode"], default="gemv")
+    ap.add_argument("--workload", choices=["gemv", "hgemm", "decode", "gemv_timeline", "gemv_grid"], default="gemv")
+    ap.add_argument("--rows", default="2048",
+                    help="--workload hgemm: row counts M of the prefill shapes that form the timed step, comma separated, "
+                         "from 16 (the four projections of a 16-token prompt), 128, 512, 2048")
+    ap.add_argument("--splitk-merge", type=int, default=0, choices=[0, 1, 2],
+                    help="--workload hgemm: where a split K is added up (tl_set_hgemm_splitk_merge): 0/2 second kernel, "
+                         "1 inside the GEMM launch")
+    ap.add_argument("--hgemm-variant", default="",
+                    help="--workload hgemm: force one kernel variant by name (tl_hgemm_variant_name), default dispatch")
     ap.add_argument("--no-extra", action="store_true", help="skip the HGEMM / per-shape / model extras")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--copy-calibration", action="store_true",
@@ -217,6 +225,97 @@ def hgemm_table(dev, randn, torch, synth, sustained_tf, shapes=None):
     return hg
 
 
+def gemv_timeline(dev, randn, torch, launches: int):
+    """Where the time of a 4096<-4096 GEMV launch goes: `launches` back-to-back launches of the stamped build of the
+    dispatch's kernel (tl_gemv_f16_stamped), each on its own matrix (> 1 GB in rotation, so W comes from HBM) and
+    its own stamp buffer.  Per launch: all workgroups started / first workgroup done / 10, 50, 90, 100 % of the
+    workgroups done, in microseconds after the first workgroup's start, and the period from one launch's first
+    start to the next one's (the share of it outside the first-start-to-last-end window is what the launch
+    boundary costs).  Medians over the launches; the GPU's constant counter ticks every 10 ns."""
+    import ctypes
+    import numpy as np
+    from tensorlib_amd._lib import check
+    N = K = 4096
+    launches = max(8, min(launches, 200))
+    nbuf = 32
+    Ws = [randn((N, K), 0.02) for _ in range(nbuf)]
+    x = randn((1, K), 1.0)
+    y = torch.empty((1, N), device="cuda", dtype=torch.float16)
+    wgs = N // 2
+    stamps = torch.zeros((launches, wgs, 2), device="cuda", dtype=torch.int64)
+    n = ctypes.c_int(0)
+
+    def run():
+        for i in range(launches):
+            check(dev.lib.tl_gemv_f16_stamped(x.data_ptr(), Ws[i % nbuf].data_ptr(), y.data_ptr(), N, K,
+                                              stamps[i].data_ptr(), 2 * wgs, ctypes.byref(n)), "tl_gemv_f16_stamped")
+    run()
+    torch.cuda.synchronize()
+    wall, ev = time_region(run, 1, torch)
+    assert n.value == wgs
+    t = stamps.cpu().numpy().astype(np.float64) * 0.01   # us
+    start, end = t[:, :, 0], t[:, :, 1]
+    first = start.min(axis=1)
+    rel_end = np.sort(end - first[:, None], axis=1)
+    rel_start = start - first[:, None]
+    q = lambda a, f: float(np.median(a[:, min(wgs - 1, int(f * wgs))]))
+    period = np.diff(first)
+    window = rel_end[:, -1]
+    return {
+        "metric": "time line of a 4096<-4096 fp16 GEMV launch (stamped build of the dispatch's kernel)",
+        "launches": launches, "workgroups": wgs, "us_per_launch_hip_events": round(ev / launches * 1e6, 2),
+        "all_workgroups_started_us": round(float(np.median(rel_start.max(axis=1))), 2),
+        "first_workgroup_done_us": round(q(rel_end, 0.0), 2),
+        "workgroups_done_us": {"10%": round(q(rel_end, 0.10), 2), "50%": round(q(rel_end, 0.50), 2),
+                               "90%": round(q(rel_end, 0.90), 2), "100%": round(float(np.median(window)), 2)},
+        "period_first_start_to_next_first_start_us": round(float(np.median(period)), 2),
+        "outside_window_us": round(float(np.median(period - window[:-1])), 2),
+        "bytes": 2 * N * K + 2 * K + 2 * N,
+        "streaming_rate_between_10_and_90_pct_GBs": round(0.8 * 2 * N * K / (q(rel_end, 0.90) - q(rel_end, 0.10)) / 1e3, 1),
+    }
+
+
+def gemv_grid_experiments(dev, randn, torch, synth):
+    """The plain streaming GEMV under capped, persistent grids and with four rows per wavefront pass, W from HBM:
+    4096<-4096 and 12288<-4096, every configuration timed over 200 launches on > 1 GB of rotating matrices."""
+    names = dev.gemv_variants()
+    out = {}
+    for (N, K) in ((4096, 4096), (12288, 4096)):
+        nbuf = max(2, int(1.0e9 // (N * K * 2)) + 1)
+        Ws = [randn((N, K), 0.02) for _ in range(nbuf)]
+        x = randn((1, K), 1.0)
+        y = torch.empty((1, N), device="cuda", dtype=torch.float16)
+        idx = [0]
+
+        def one():
+            dev.matmul2d(x, Ws[idx[0] % nbuf], y)
+            idx[0] += 1
+        rows = {}
+        configs = [("dispatch (2 rows per pass, one row block per workgroup)", 0, 0)]
+        v2, v4 = names.index("stream_w4r2u2s4x1"), names.index("stream_w4r4u2s4x1")
+        for k in (2, 4, 8):
+            configs.append((f"2 rows per pass, grid capped at {k} workgroups per CU (persistent)", v2, 4 * k))
+        configs.append(("4 rows per pass, one row block per workgroup", v4, 1 << 20))
+        for k in (2, 4, 8):
+            configs.append((f"4 rows per pass, grid capped at {k} workgroups per CU (persistent)", v4, 4 * k))
+        for name, variant, wpc in configs:
+            dev.set_gemv_variant(variant)
+            dev.lib.tl_set_gemv_grid_waves_per_cu(wpc)
+            best = None
+            for _ in range(3):
+                for _ in range(10):
+                    one()
+                _, ev = time_region(one, 200, torch)
+                us = ev / 200 * 1e6
+                best = us if best is None else min(best, us)
+            rows[name] = {"us": round(best, 2), "frac_hbm": round(synth.gemv_bytes(N, K) / best / 1e3 / HBM_PEAK_GBS, 4)}
+        dev.set_gemv_variant(0)
+        dev.lib.tl_set_gemv_grid_waves_per_cu(0)
+        out[f"{N}x{K}"] = rows
+        del Ws
+    return {"metric": "fp16 GEMV grid experiments (us per launch, best of 3 x 200 launches, W from HBM)", "results": out}
+
+
 def main():
     args = parse_args()
     if args.gpus != 1:
@@ -264,8 +363,23 @@ def main():
         print(json.dumps(out))
         return
 
+    if args.workload == "gemv_timeline":
+        print(json.dumps(gemv_timeline(dev, randn, torch, args.steps)))
+        return
+    if args.workload == "gemv_grid":
+        print(json.dumps(gemv_grid_experiments(dev, randn, torch, synth)))
+        return
+
     if args.workload == "hgemm":
-        shapes = [s for s in HGEMM_SHAPES if s[0] == 2048]
+        rows = [int(r) for r in args.rows.split(",")]
+        short_prompt = [(16, 12288, 4096), (16, 4096, 4096), (16, 22016, 4096), (16, 4096, 11008)]
+        shapes = [s for s in HGEMM_SHAPES + short_prompt if s[0] in rows]
+        if not shapes:
+            print(f"--rows {args.rows}: no prefill shape has that many rows", file=sys.stderr)
+            sys.exit(2)
+        dev.lib.tl_set_hgemm_splitk_merge(args.splitk_merge)
+        if args.hgemm_variant:
+            dev.set_hgemm_variant(dev.hgemm_variants().index(args.hgemm_variant))
         mats = [(randn((M, K), 1.0), randn((N, K), 0.02), torch.empty((M, N), device="cuda", dtype=torch.float16))
                 for (M, N, K) in shapes]
         step_flops = sum(synth.gemm_flops(*s) for s in shapes)
@@ -280,12 +394,13 @@ def main():
         achieved = step_flops / (ev / args.steps) / 1e12
         sustained = mfma_sustained(dev)
         out = {
-            "metric": "fp16 HGEMM TFLOP/s (Llama2-7B prefill, M=2048 shapes)",
+            "metric": f"fp16 HGEMM TFLOP/s (Llama2-7B prefill, M={args.rows} shapes)",
             "value": round(value, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
             "ms_per_step": round(wall * 1e3 / args.steps, 5), "higher_is_better": True, "scaling": "weak",
             "vs_baseline": None, "dtype": "f16", "data": "synthetic",
-            "config": {"workload": "prefill HGEMM X[2048,K] . W[N,K]^T for (N,K) in 4096x4096, 11008x4096, 32000x4096, "
-                                   "4096x11008; X~N(0,1), W~N(0,0.02); fp32 accumulate", "flops_per_step": step_flops},
+            "config": {"workload": "prefill HGEMM X[M,K] . W[N,K]^T for (M,N,K) in " + ", ".join("x".join(map(str, s)) for s in shapes) +
+                                   "; X~N(0,1), W~N(0,0.02); fp32 accumulate", "flops_per_step": step_flops,
+                       "splitk_merge": args.splitk_merge, "variant": args.hgemm_variant or "dispatch"},
             "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": MFMA_FP16_PEAK_TFLOPS, "unit": "TFLOP/s",
                          "frac": round(achieved / MFMA_FP16_PEAK_TFLOPS, 4), "traffic": None,
                          "kernel": "hgemm_f16_dlds_kernel", "flops_per_launch": step_flops / len(shapes),
@@ -293,7 +408,7 @@ def main():
                          "sustained_mfma_tflops": sustained},
         }
         if not args.no_extra:
-            out["extra"] = {"hgemm_prefill": hgemm_table(dev, randn, torch, synth, sustained["changing_operands"])}
+            out["extra"] = {"hgemm_prefill": hgemm_table(dev, randn, torch, synth, sustained["changing_operands"], shapes)}
         if not args.no_cpu:
             out["cpu_baseline"] = cpu_baseline_hgemm()
         print(json.dumps(out))

@@ -52,7 +52,11 @@ const char* tl_version(void);
 int tl_device_cu_count(void);
 
 /* Enqueue all later work on `hip_stream` (a hipStream_t; NULL = null stream).
- * The reference uses the default stream everywhere (tensorLib/src/device/cuda/gemm.cu). */
+ * The reference uses the default stream everywhere (tensorLib/src/device/cuda/gemm.cu).
+ * When the stream changes and the stream being replaced has used the library's scratch buffers (split-K GEMM,
+ * decode attention with more than one chunk), this call waits for that stream to drain, so the buffers are free
+ * when the first call on the new stream reuses them; the stream being replaced must therefore still exist when
+ * this is called, and may be destroyed right after. */
 int tl_set_stream(void* hip_stream);
 void* tl_get_stream(void);
 
@@ -67,6 +71,14 @@ int tl_memcpy_h2d(void* dst, const void* host_src, size_t bytes);
 int tl_memcpy_d2h(void* host_dst, const void* src, size_t bytes);
 int tl_memcpy_d2d(void* dst, const void* src, size_t bytes);
 int tl_synchronize(void);
+
+/* Zeroes the counters the library keeps in its own device scratch between calls: the per-head tickets of the decode
+ * attention (grown-on-demand workspace and static array) and the per-tile tickets of the one-launch split-K GEMM.
+ * Every kernel leaves them at zero when it completes, so this is only needed after a launch that did not complete
+ * (a device error reported by a later call, a stream destroyed with work pending): a ticket left set would make
+ * later calls merge early, silently.  Enqueues fill kernels on the library's stream; no allocation, no host wait.
+ * No counterpart in the reference (its kernels keep no state between launches). */
+int tl_reset_scratch(void);
 
 /* ------------------------------------------------------- the hot path ---- */
 
@@ -107,14 +119,30 @@ int tl_set_hgemm_variant(int variant);
 const char* tl_gemv_variant_name(int variant);
 const char* tl_hgemm_variant_name(int variant);
 /* Measurement hook (no reference counterpart): fp16 MFMA rate sustained out of registers, in
- * TFLOP/s.  mode 0: constant operands; mode 1: both operands change with every instruction.
+ * TFLOP/s.  mode 0: constant operands; mode 1: both operands change with every instruction (v_mfma_f32_32x32x16_f16);
+ * modes 2 and 3: the same two with v_mfma_f32_16x16x32_f16.
  * Synchronises the stream.  Used by bench.py to place HGEMM against the power-managed ceiling. */
 int tl_measure_mfma_rate_f16(int mode, double* tflops);
+/* Measurement hook (no reference counterpart): the GEMV kernel the dispatch uses for K <= 4096, built with time stamps.
+ * Same arithmetic and stores as tl_gemv_f16; in addition workgroup g writes the GPU's constant 100 MHz counter at its
+ * first instruction to stamps[2 g] and after its last store to stamps[2 g + 1] (device memory, uint64, capacity in
+ * elements); *workgroups receives the number of workgroups launched.  bench.py --workload gemv_timeline turns the
+ * stamps of a sequence of launches into the launch time line (ramp, streaming phase, tail, time between launches). */
+int tl_gemv_f16_stamped(const void* x, const void* W, void* y, size_t N, size_t K, void* stamps,
+                        size_t stamps_capacity, int* workgroups);
 /* Tuning hook: force the number of K splits of the MFMA GEMM (0 = automatic). */
 int tl_set_hgemm_splits(int splits);
 /* Inspection hook (no reference counterpart): the kernel variant (index into tl_hgemm_variant_name(); -1 = the
  * kernel for at most 32 rows) and the number of K splits the most recent fp16 GEMM launch of this process used. */
 int tl_hgemm_last_plan(int* variant, int* splits);
+/* Tuning hook: where the fp32 partial sums of a split-K GEMM are added up.  0 = automatic and 2 = by a second kernel
+ * (the default: measured faster on every split shape); 1 = inside the GEMM launch, by the workgroup that finishes a
+ * C tile's last split (one counter per tile in the library's scratch, zero between launches), whenever C takes 8-byte
+ * stores (N % 8 == 0, 16-byte aligned C), the tile is at most 128x256, the launch has at most 4096 tiles and the
+ * partial sums stay below 2 GiB, else the second kernel.  Both add the splits in split order: same bits.
+ * tl_hgemm_last_split_in_launch() tells which one the most recent GEMM launch used (1 = inside the launch). */
+int tl_set_hgemm_splitk_merge(int mode);
+int tl_hgemm_last_split_in_launch(void);
 /* Tuning hook: the MFMA GEMM's workgroups start their walk over K at K tile
  * (tile_column * per_tile + xcd * per_xcd) % tiles and wrap (-1 = automatic, 0 = no rotation). */
 int tl_set_hgemm_k_rotation(int per_tile, int per_xcd);
@@ -129,7 +157,9 @@ int tl_set_hgemm_fewrows(int mode);
 int tl_set_prefill_attention_variant(int variant);
 /* Tuning hook: where the chunk partials of the decode attention are merged: 0 = automatic (inside the one launch
  * up to 512 cached positions), 1 = always inside the launch, by the workgroup that finishes a head's last chunk,
- * 2 = always by a second launch.  Same bits either way. */
+ * 2 = always by a second launch, 3 = like 1 but ordered by a release/acquire read-modify-write on the ticket and plain
+ * accesses to the partials (the HIP memory model's own terms; slower, kept as the tested alternative).  Same bits
+ * in every mode. */
 int tl_set_decode_attention_merge(int mode);
 /* Tuning hook: cached positions per workgroup of the decode attention: 0 = automatic, else 64, 128 or 256
  * (head_dim 256 always uses 64). */
@@ -237,13 +267,15 @@ int tl_decode_attention_rope_f16(void* out, const void* qkv, void* cache_k, void
  * results; the per-chunk partial results go to a static device array of TL_DECODE_ATTENTION_STATIC_SCRATCH_FLOATS
  * floats that is part of the library's code object (each GPU holds its copy until the process ends) instead of the
  * grown-on-demand workspace, and the call makes no hipMalloc / hipFree.  Limit:
- *   64 * ceil(n_heads / 64) + n_heads * ceil((pos + 1) / 64) * (head_dim + 2) <= TL_DECODE_ATTENTION_STATIC_SCRATCH_FLOATS
- * (32 heads of 128: 16128 positions) is always accepted; what exceeds the array returns TL_EINVAL (contexts from 1280
+ *   1024 + n_heads * ceil((pos + 1) / 64) * (head_dim + 2) <= TL_DECODE_ATTENTION_STATIC_SCRATCH_FLOATS
+ * (32 heads of 128: 16064 positions) is always accepted; what exceeds the array returns TL_EINVAL (contexts from 1280
  * positions on with head_dim up to 128 are cut into chunks of 128 positions and need half of that).  Every call on a GPU shares that GPU's array:
  * calls that overlap on one GPU (two streams, two host threads) race; calls on one stream do not.  The caller clears
- * nothing: every partial a call reads was written by the same call, and the per-head tickets at the head of the array
- * (64 words per 64 heads, counted in the limit) are zero when the library is loaded and are set back to zero by the
- * workgroup that draws a head's last one. */
+ * nothing: every partial a call reads was written by the same call, and the per-head tickets in the first 1024 words
+ * of the array (one per head whatever the head count; launches with more than 1024 heads merge with a second kernel
+ * and use none) are zero when the library is loaded and are set back to zero by the workgroup that draws a head's
+ * last one.  Only a launch that did not run to completion (a device error, a process that tore the stream down)
+ * can leave a ticket set; tl_reset_scratch() clears them. */
 #define TL_DECODE_ATTENTION_STATIC_SCRATCH_FLOATS (1u << 20)
 int tl_decode_attention_rope_static_f16(void* out, const void* qkv, void* cache_k, void* cache_v,
                                         const void* rope_table, int pos, int n_heads, int head_dim);

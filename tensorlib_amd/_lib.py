@@ -52,9 +52,11 @@ _PROTOS = {
     "tl_memcpy_d2h": (_i, [_vp, _vp, _sz]),
     "tl_memcpy_d2d": (_i, [_vp, _vp, _sz]),
     "tl_synchronize": (_i, []),
+    "tl_reset_scratch": (_i, []),
     "tl_matmul2d_f16": (_i, [_vp, _vp, _vp, _sz, _sz, _sz]),
     "tl_gemv_f16": (_i, [_vp, _vp, _vp, _sz, _sz]),
     "tl_hgemm_f16": (_i, [_vp, _vp, _vp, _sz, _sz, _sz]),
+    "tl_gemv_f16_stamped": (_i, [_vp, _vp, _vp, _sz, _sz, _vp, _sz, _ip]),
     "tl_hgemm_silu_mul_f16": (_i, [_vp, _vp, _vp, _vp, _sz, _sz, _sz]),
     "tl_matmul2d_batched_f16": (_i, [_vp, _vp, _vp, _sz, _sz, _sz, _sz, _sz, _sz, _sz]),
     "tl_matmul2d_f32": (_i, [_vp, _vp, _vp, _sz, _sz, _sz]),
@@ -64,6 +66,8 @@ _PROTOS = {
     "tl_hgemm_variant_name": (_c.c_char_p, [_i]),
     "tl_set_gemv_grid_waves_per_cu": (_i, [_i]),
     "tl_set_hgemm_splits": (_i, [_i]),
+    "tl_set_hgemm_splitk_merge": (_i, [_i]),
+    "tl_hgemm_last_split_in_launch": (_i, []),
     "tl_hgemm_last_plan": (_i, [_c.POINTER(_c.c_int), _c.POINTER(_c.c_int)]),
     "tl_set_hgemm_k_rotation": (_i, [_i, _i]),
     "tl_set_hgemm_tile_band": (_i, [_i]),

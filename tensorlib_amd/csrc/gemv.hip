@@ -95,6 +95,9 @@ struct GemvArgs {
     const half8_t* g;   // norm weight
     half8_t* sum_out;   // may be null; receives half(x + x2), written by workgroup 0
     float eps;
+    // stamped build of the streaming kernel only: stamps[2 * workgroup] / [2 * workgroup + 1] receive the constant
+    // 100 MHz counter (s_memrealtime) at the workgroup's first instruction and after its last store
+    unsigned long long* stamps;
 };
 
 // One wavefront per row group.  Dynamic LDS: K8 chunks of x (+ partial sums when KSPLIT > 1).
@@ -204,11 +207,15 @@ __global__ void __launch_bounds__(WAVES * 64) gemv_f16_wave_kernel(GemvArgs a) {
 //            Workgroup 0 also writes half(h + d) out (the new residual stream).
 // Dynamic LDS: [K8 chunks of x when XMODE == 0] + 2*RG*KSPLIT*ROWS floats when KSPLIT > 1
 //              (+ WAVES floats when XMODE == 3).
-template <int WAVES, int ROWS, int UNROLL, int KSPLIT, int XMODE>
+// STAMP: measurement build (tl_gemv_f16_stamped): thread 0 of every workgroup records the time at its first
+// instruction and after the workgroup's last store; otherwise the same instructions.
+template <int WAVES, int ROWS, int UNROLL, int KSPLIT, int XMODE, bool STAMP = false>
 __global__ void __launch_bounds__(WAVES * 64) gemv_f16_stream_kernel(GemvArgs a) {
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
     half8_t* xs = reinterpret_cast<half8_t*>(smem_raw);
 
+    unsigned long long t_start = 0;
+    if constexpr (STAMP) t_start = __builtin_amdgcn_s_memrealtime();
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = tid >> 6;
@@ -356,6 +363,14 @@ __global__ void __launch_bounds__(WAVES * 64) gemv_f16_stream_kernel(GemvArgs a)
             for (int r = 0; r < ROWS; ++r)
 #pragma unroll
                 for (int u = 0; u < UNROLL; ++u) cur[r][u] = nxt[r][u];
+        }
+    }
+    if constexpr (STAMP) {
+        __syncthreads();   // the wavefronts that wrote y have passed their stores
+        if (tid == 0) {
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            a.stamps[2 * blockIdx.x] = t_start;
+            a.stamps[2 * blockIdx.x + 1] = __builtin_amdgcn_s_memrealtime();
         }
     }
 }
@@ -514,6 +529,7 @@ int launch_gemv(const void* x, const void* W, void* y, size_t N, size_t K, size_
     a.g = norm ? (const half8_t*)norm->weight : nullptr;
     a.sum_out = norm ? (half8_t*)norm->sum_out : nullptr;
     a.eps = norm ? norm->eps : 0.f;
+    a.stamps = nullptr;
 
     const int forced_variant = g_forced_variant.load();
     if (a.K8 < 64 && forced_variant == 0) {
@@ -623,6 +639,32 @@ int tl_set_gemv_grid_waves_per_cu(int waves) {
 }
 
 }  // extern "C"
+
+// The dispatch's kernel for K <= 4096 (<4,2,2,4,1>, one row block per workgroup) in its stamped build.
+extern "C" int tl_gemv_f16_stamped(const void* x, const void* W, void* y, size_t N, size_t K, void* stamps,
+                                   size_t stamps_capacity, int* workgroups) {
+    TL_ENSURE_INIT();
+    TL_REQUIRE(x && W && y && stamps && workgroups, "tl_gemv_f16_stamped: null pointer");
+    TL_REQUIRE(K % 8 == 0 && K >= 512 && K <= 4096 && tl::aligned16(x) && tl::aligned16(W) && N >= 1 && N <= 0x7fffffffu,
+               "tl_gemv_f16_stamped: needs 512 <= K <= 4096, K %% 8 == 0 and 16-byte aligned operands");
+    constexpr int WAVES = 4, ROWS = 2, KSPLIT = 4;
+    tl::GemvArgs a{};
+    a.x = (const tl::half8_t*)x;
+    a.W = (const tl::half8_t*)W;
+    a.y = (tl::half_t*)y;
+    a.N = (int)N;
+    a.K8 = (int)(K / 8);
+    a.num_row_blocks = (int)((N + ROWS - 1) / ROWS);
+    a.stamps = (unsigned long long*)stamps;
+    TL_REQUIRE((size_t)a.num_row_blocks * 2 <= stamps_capacity, "tl_gemv_f16_stamped: %d workgroups need %d stamps, the buffer holds %zu",
+               a.num_row_blocks, 2 * a.num_row_blocks, stamps_capacity);
+    *workgroups = a.num_row_blocks;
+    const size_t lds = (size_t)2 * (WAVES / KSPLIT) * KSPLIT * ROWS * 4;
+    hipLaunchKernelGGL((tl::gemv_f16_stream_kernel<WAVES, ROWS, 2, KSPLIT, 1, true>), dim3(a.num_row_blocks), dim3(WAVES * 64), lds,
+                       tl::stream(), a);
+    TL_CHECK_LAUNCH("gemv_f16_stream_kernel<stamped>");
+    return TL_OK;
+}
 
 extern "C" int tl_gemv_silu_mul_f16(const void* ab, const void* W, void* y, size_t N, size_t K) {
     TL_ENSURE_INIT();

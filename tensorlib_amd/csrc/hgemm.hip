@@ -22,58 +22,11 @@
 #include <numeric>
 #include <type_traits>
 
-#include "tl_internal.h"
+#include "hgemm_common.h"
 
 namespace tl {
 
-struct HgemmArgs {
-    const half_t* A;
-    const half_t* B;
-    half_t* C;
-    int M, N, K;
-    int ldc;  // elements between rows of C (N, unless the launch covers a column range of a wider C)
-    int tiles_m, tiles_n;
-    long sa, sb, sc;  // batch strides in elements
-    // split-K (direct-to-LDS kernel only): blockIdx.z walks K tiles [z*kt_per_split, ...) and writes
-    // fp32 partial sums to partial[z][M][N]; a second kernel adds the splits in order.
-    int kt_per_split;
-    float* partial;
-    // K rotation: a workgroup walks its K tiles starting at (tile_n * rot_tile + xcd * rot_xcd) % KT and wraps.
-    // Workgroups that run at the same time then touch different column offsets of the 8 KB-strided rows, which
-    // spreads their requests over the memory channels (tile-shaped streaming of B from HBM: 4.3 -> 5.9 TB/s).
-    int rot_tile, rot_xcd;
-    // Tiles are numbered band by band: a band is band_m rows of tiles over all columns, walked column by column.
-    int band_m;
-    // Gated launches (kernels built with MODE 2): B holds two matrices `gate` rows apart, N counts the rows of both
-    // (2 x the output columns), and C[m][n] = silu(A[m,:].B[n,:]) * (A[m,:].B[gate + n,:]) for n < N / 2.
-    int gate;
-};
-
 constexpr int kPad = 8;  // halves of padding per LDS row
-
-// Map the linear workgroup id to a tile so that workgroups resident on one XCD (ids
-// congruent mod 8 are dispatched to the same XCD) work on neighbouring tiles: XCD x takes a contiguous run of
-// tile numbers, and tiles are numbered down a band of `band` rows of tiles, column after column, band after
-// band.  The 32 tiles an XCD works on at a time then cover about band x 32/band panels of A and B, which its
-// L2 serves to all of them; with more rows of tiles than `band` a whole column of tiles would share only its
-// panel of B and pull every panel of A through the L2 for a single use.
-__device__ __forceinline__ void tile_of_block(int bid, int nblocks, int tiles_m, int band, int& tm, int& tn) {
-    // nblocks / 8 tiles per XCD, one more on the first nblocks % 8 XCDs
-    const int x = bid & 7, base = nblocks >> 3, rem = nblocks & 7;
-    const int lid = x * base + (x < rem ? x : rem) + (bid >> 3);
-    if (band >= tiles_m) {
-        tm = lid % tiles_m;
-        tn = lid / tiles_m;
-        return;
-    }
-    const int tiles_n = nblocks / tiles_m;
-    const int per_band = band * tiles_n;
-    const int b = lid / per_band;
-    const int r = lid - b * per_band;
-    const int rows = (tiles_m - b * band) < band ? (tiles_m - b * band) : band;  // the last band may be lower
-    tm = b * band + r % rows;
-    tn = r / rows;
-}
 
 template <int BM, int BN, int BK, int WM, int WN>
 __global__ void __launch_bounds__(WM* WN * 64) hgemm_f16_mfma_kernel(HgemmArgs a) {
@@ -237,6 +190,9 @@ __global__ void __launch_bounds__(WM* WN * 64) hgemm_f16_dlds_kernel(HgemmArgs a
     constexpr int MT = TM / 32, NT = TN / 32;
     constexpr int KS = BK / 16;
     constexpr bool GATED = MODE == 2;
+    // the in-launch merge of split-K is compiled for tiles up to 128x256 (the ones a split launch uses; in the 256x256
+    // kernels its registers would add to a budget that is already full)
+    constexpr bool TICKETS = BM * BN <= 128 * 256;
     static_assert(!GATED || TN % 16 == 0, "a wavefront column holds two halves of whole 16-byte pieces");
     static_assert(BK == 32 || BK == 64, "BK must be 32 or 64");
     static_assert(BM % (RPW * NW) == 0 && BN % (RPW * NW) == 0, "tile rows must split over the wavefronts");
@@ -268,12 +224,13 @@ __global__ void __launch_bounds__(WM* WN * 64) hgemm_f16_dlds_kernel(HgemmArgs a
     // loop would make the compiler treat lgkmcnt as unordered and turn every wait for LDS data into
     // lgkmcnt(0), which also waits for the fragment reads issued just before it.
     float* const partial = a.partial;
+    unsigned* const tickets = a.tickets;
     const int ldc = a.ldc;
     const unsigned rot_tile = (unsigned)a.rot_tile, rot_xcd = (unsigned)a.rot_xcd;
     const int band_m = a.band_m;
     const int gate = GATED ? a.gate : 0;
     asm volatile("" ::"s"(partial), "s"(C), "s"(M), "s"(N), "s"(a.kt_per_split), "s"(rot_tile), "s"(rot_xcd), "s"(band_m), "s"(ldc),
-                 "s"(gate));
+                 "s"(gate), "s"(tickets));
 
     // ---- loader: wavefront-load j of this wavefront covers tile rows (j*NW + wave)*RPW .. +RPW ----
     // A request's address is a wavefront-uniform base (first row of the tile at the K tile wanted, in scalar
@@ -511,6 +468,7 @@ __global__ void __launch_bounds__(WM* WN * 64) hgemm_f16_dlds_kernel(HgemmArgs a
     const int e_row = lane & 31;
     const int e_col = (lane >> 5) * 4;
     const int row_base = m0 + wm * TM, col_base = GATED ? n0 + wn * (TN / 2) : n0 + wn * TN;
+    const int tile_m0 = m0, tile_n0 = n0;   // setup_tile() moves m0 and n0 on to the next tile before the stores
     constexpr int RS = TN * 2 + 16;          // bytes per staged row of the fp16 epilogue
     // (a gated launch is always staged: the host launches it only for 16-byte aligned rows of C and without split)
     const bool staged = GATED || (!partial && (N % 8) == 0 && (ldc % 8) == 0 && (reinterpret_cast<uintptr_t>(C) & 15u) == 0);
@@ -566,8 +524,92 @@ __global__ void __launch_bounds__(WM* WN * 64) hgemm_f16_dlds_kernel(HgemmArgs a
                 *reinterpret_cast<half8_t*>(C + (size_t)row * ldc + col) = o;
             }
         }
+    } else if (TICKETS && partial && tickets) {
+        // split-K in one launch.  The fp32 partial sums of this split leave as device-coherent 16-byte stores (sc1:
+        // written through to the level all XCDs share); every wavefront waits until its stores are acknowledged,
+        // the workgroup barrier collects those waits, and then one thread draws the tile's ticket with a
+        // device-scope atomic.  The workgroup that draws the last ticket of a tile reads all slabs of the tile back
+        // with device-coherent loads, adds them in split order, exactly the sum and rounding of
+        // splitk_reduce_kernel, writes fp16 C and sets the ticket back to zero for the next launch.  The ring is
+        // drained at this point, so the waits cost nothing that the epilogue would not have waited for anyway.
+        // The host guarantees N % 8 == 0, 16-byte aligned C and slabs, and byte offsets below 2^31.
+        typedef unsigned u32x4_t __attribute__((ext_vector_type(4)));
+        const unsigned slab_bytes = (unsigned)M * (unsigned)N * 4u;
+        const __amdgpu_buffer_rsrc_t slabs = __builtin_amdgcn_make_buffer_rsrc(partial, 0, (int)(slab_bytes * gridDim.z), 0x00020000);
+        constexpr int kCoherent = 16;   // sc1
+#pragma unroll
+        for (int i = 0; i < MT; ++i) {
+            const int row = row_base + i * 32 + e_row;
+            const unsigned row_off = (unsigned)blockIdx.z * slab_bytes + (unsigned)row * (unsigned)N * 4u;
+#pragma unroll
+            for (int j = 0; j < NT; ++j)
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    const int col = col_base + j * 32 + g * 8 + e_col;
+                    if (row < M && col < N) {
+                        float4_t v = {acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]};
+                        __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4_t, v), slabs, (int)(row_off + (unsigned)col * 4u), 0, kCoherent);
+                    }
+                }
+        }
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+        volatile int* flag = reinterpret_cast<volatile int*>(smem_raw + stage_area);
+        if (tid == 0) {
+            const unsigned t = __hip_atomic_fetch_add(tickets + vb, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            const int last = (t + 1u == gridDim.z);
+            if (last) __hip_atomic_store(tickets + vb, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            *flag = last;
+        }
+        __syncthreads();
+        const bool merge = *flag != 0;
+        __syncthreads();   // the flag's word belongs to the next tile's ring once this workgroup moves on
+        if (merge) {
+            constexpr int C4 = BN / 4, THREADS = NW * 64, ITEMS = BM * C4 / THREADS, U = ITEMS < 4 ? ITEMS : 4;
+            static_assert(BM * C4 % THREADS == 0 && ITEMS % U == 0, "tile must split evenly over the threads");
+            const int splits = (int)gridDim.z;
+            for (int it0 = 0; it0 < ITEMS; it0 += U) {
+                float4_t sum[U];
+                unsigned off[U];
+                bool ok[U];
+#pragma unroll
+                for (int u = 0; u < U; ++u) {
+                    const int idx = (it0 + u) * THREADS + tid;
+                    const int row = tile_m0 + idx / C4, col = tile_n0 + (idx % C4) * 4;
+                    ok[u] = row < M && col < N;
+                    off[u] = ok[u] ? ((unsigned)row * (unsigned)N + (unsigned)col) * 4u : 0u;
+                }
+                for (int s0 = 0; s0 < splits; s0 += 4) {
+                    u32x4_t v[4][U];
+#pragma unroll
+                    for (int k = 0; k < 4; ++k)
+                        if (s0 + k < splits) {
+#pragma unroll
+                            for (int u = 0; u < U; ++u)
+                                v[k][u] = __builtin_amdgcn_raw_buffer_load_b128(slabs, (int)(off[u] + (unsigned)(s0 + k) * slab_bytes), 0, kCoherent);
+                        }
+#pragma unroll
+                    for (int k = 0; k < 4; ++k)
+                        if (s0 + k < splits) {
+#pragma unroll
+                            for (int u = 0; u < U; ++u) {
+                                const float4_t f = __builtin_bit_cast(float4_t, v[k][u]);
+                                sum[u] = (s0 + k == 0) ? f : sum[u] + f;
+                            }
+                        }
+                }
+#pragma unroll
+                for (int u = 0; u < U; ++u) {
+                    if (!ok[u]) continue;
+                    const int idx = (it0 + u) * THREADS + tid;
+                    const int row = tile_m0 + idx / C4, col = tile_n0 + (idx % C4) * 4;
+                    half4_t h = {(half_t)sum[u][0], (half_t)sum[u][1], (half_t)sum[u][2], (half_t)sum[u][3]};
+                    *reinterpret_cast<half4_t*>(C + (size_t)row * ldc + col) = h;
+                }
+            }
+        }
     } else if (partial) {
-        // split-K: fp32 partial sums, four consecutive columns (16 bytes) per store where the row allows it
+        // split-K with a second kernel: fp32 partial sums, four consecutive columns (16 bytes) per store where the row allows it
         const bool vec = (N % 4) == 0;
 #pragma unroll
         for (int i = 0; i < MT; ++i) {
@@ -735,6 +777,9 @@ static const HgemmVariant g_variants[] = {
     TL_HGEMM_PIPE(256, 192, 64, 2, 2, 2),  // 18
     // few rows: four wavefronts of 64x64 read a quarter fewer fragment bytes from LDS than eight of 64x32
     TL_HGEMM_PIPE(128, 128, 64, 2, 2, 4),  // 19
+    // hgemm_vstage.hip: one wavefront per SIMD, accumulators in AGPRs, two K tiles in flight in registers (stages < 0:
+    // index -stages - 1 into that file's table)
+    {"v256x256x64w2x2", 256, 256, 64, 256, -1, nullptr, true, nullptr},  // 20
 };
 
 static constexpr int kNumVariants = sizeof(g_variants) / sizeof(g_variants[0]);
@@ -744,8 +789,16 @@ static std::atomic<bool> g_attr_set[kNumVariants], g_attr_set_gated[kNumVariants
 
 static std::atomic<int> g_forced_splits{0};  // 0 = automatic
 static std::atomic<int> g_last_variant{0}, g_last_splits{0};   // what the most recent tile launch used
+static std::atomic<bool> g_last_one_launch{false};             // its split-K was merged inside the launch
 static std::atomic<int> g_forced_rot_tile{-1}, g_forced_rot_xcd{-1};  // -1 = automatic
 static std::atomic<int> g_forced_band{0};                              // 0 = automatic
+// Where the slabs of a split K are added up: 0 = automatic = 2 = by the second kernel; 1 = inside the GEMM launch, by the
+// workgroup that finishes a tile's last split.  The second kernel is the default because it is faster (same box, W from
+// HBM, second kernel against in-launch: 128x4096x4096 15.2 / 17.0 us, 128x11008x4096 29.9 / 36.1, 128x4096x11008
+// 32.2 / 36.3, 256x4096x11008 40.8 / 47.2, 512x4096x11008 60.8 / 69.4): the slabs have to leave as write-through
+// stores and come back through device-coherent loads, a serial chain of store acknowledgement, ticket and reload of
+// about 4 us at the end of every tile, where the second kernel reads slabs that still sit in the L2s with every CU.
+static std::atomic<int> g_splitk_merge_mode{0};
 
 // Library-owned fp32 workspace for split-K partial sums, grown on demand (stream-ordered reuse).
 static Workspace g_splitk;
@@ -965,6 +1018,21 @@ static int launch_hgemm_cols(const void* A, const void* B, void* C, size_t M, si
         static const int v_square = hgemm_variant_index("p128x128x64w2x2s4");
         if (square_splits > 0) vi = v_square;
     }
+    if (g_variants[vi].stages < 0) {
+        // the register-staged kernel: one dense fp16 C, no gate, no split; anything else falls back to the ring kernel
+        const int forced_band = g_forced_band.load();
+        const int KTv = (int)(K / 64);
+        const int rt = g_forced_rot_tile.load(), rx = g_forced_rot_xcd.load();
+        if (gate == 0 && batch == 1 && hgemm_vstage_applies(A, B, C, M, N, K, ldc)) {
+            g_last_variant = vi;
+            g_last_splits = 1;
+            g_last_one_launch = false;
+            return launch_hgemm_vstage(-g_variants[vi].stages - 1, A, B, C, M, N, K, ldc, forced_band > 0 ? forced_band : 8,
+                                       rt >= 0 ? rt : 0, rx >= 0 ? rx : KTv / 8);
+        }
+        static const int v_big = hgemm_variant_index("p256x256x64w2x4s2");
+        vi = v_big;
+    }
     if (g_variants[vi].stages > 0 && K % g_variants[vi].bk != 0) vi = 1;  // direct-to-LDS path cannot zero-fill a K tail
     // its per-lane byte offsets inside a tile ((rows - 1) * K + 64 halves) are 32-bit
     if (g_variants[vi].stages > 0 && K > ((size_t)1 << 22)) vi = 1;
@@ -1002,6 +1070,7 @@ static int launch_hgemm_cols(const void* A, const void* B, void* C, size_t M, si
     TL_REQUIRE(nblocks <= 0x7fffffffu, "hgemm: too many tiles");
     a.kt_per_split = 0x7fffffff;
     a.partial = nullptr;
+    a.tickets = nullptr;
     a.rot_tile = 0;
     a.rot_xcd = 0;
     a.gate = (int)gate;
@@ -1035,9 +1104,16 @@ static int launch_hgemm_cols(const void* A, const void* B, void* C, size_t M, si
         if (splits > 1) {
             a.kt_per_split = (KT + splits - 1) / splits;
             splits = (KT + a.kt_per_split - 1) / a.kt_per_split;
-            int rc = g_splitk.acquire((size_t)splits * M * N, (size_t)8 << 20, "split-K workspace", &lease);
+            // [kSplitkTicketWords tile tickets][splits x M x N floats]
+            int rc = g_splitk.acquire(kSplitkTicketWords + (size_t)splits * M * N, (size_t)8 << 20, "split-K workspace", &lease);
             if (rc != TL_OK) return rc;
-            a.partial = lease.ptr;
+            a.partial = lease.ptr + kSplitkTicketWords;
+            // the last workgroup of a tile adds the slabs itself unless the caller folds that pass into its own kernel,
+            // there are more tiles than tickets, or C cannot take its 8-byte stores / the slabs exceed 32-bit offsets
+            const bool one_launch = !(partials_out && splits_out) && g_splitk_merge_mode.load() == 1 &&
+                                    nblocks <= kSplitkTicketWords && N % 8 == 0 && aligned16(C) && v.bm * v.bn <= 128 * 256 &&
+                                    (size_t)splits * M * N * sizeof(float) < ((size_t)1 << 31);
+            if (one_launch) a.tickets = reinterpret_cast<unsigned*>(lease.ptr);
         }
     }
     g_last_variant = vi;
@@ -1070,7 +1146,8 @@ static int launch_hgemm_cols(const void* A, const void* B, void* C, size_t M, si
         *splits_out = splits;
         return TL_OK;
     }
-    if (splits > 1) {
+    g_last_one_launch = a.tickets != nullptr;
+    if (splits > 1 && !a.tickets) {
         const size_t n = M * N;
         size_t blocks = (n / 4 + 255) / 256;
         const size_t cap = (size_t)device_info().cu_count * 8;
@@ -1081,6 +1158,8 @@ static int launch_hgemm_cols(const void* A, const void* B, void* C, size_t M, si
     }
     return TL_OK;
 }
+
+int splitk_reset_tickets() { return g_splitk.zero_head(kSplitkTicketWords); }
 
 // One launch can apply the gate when the pipelined kernels serve the shape (K in whole tiles of 64, lane offsets within
 // 32 bits over both matrices), C takes 16-byte stores, and no variant without a gated build is forced.
@@ -1169,6 +1248,14 @@ int tl_set_hgemm_tile_band(int band) {
     tl::g_forced_band = band;
     return TL_OK;
 }
+
+int tl_set_hgemm_splitk_merge(int mode) {
+    TL_REQUIRE(mode >= 0 && mode <= 2, "tl_set_hgemm_splitk_merge: %d out of range [0,2]", mode);
+    tl::g_splitk_merge_mode = mode;
+    return TL_OK;
+}
+
+int tl_hgemm_last_split_in_launch(void) { return tl::g_last_one_launch.load() ? 1 : 0; }
 
 int tl_hgemm_last_plan(int* variant, int* splits) {
     TL_REQUIRE(variant && splits, "tl_hgemm_last_plan: null output");

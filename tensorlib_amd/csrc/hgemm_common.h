@@ -1,0 +1,65 @@
+// Shared by the translation units that hold the fp16 tile GEMM kernels: the kernel argument block and the
+// workgroup-to-tile map.
+#pragma once
+#include "tl_internal.h"
+
+namespace tl {
+
+struct HgemmArgs {
+    const half_t* A;
+    const half_t* B;
+    half_t* C;
+    int M, N, K;
+    int ldc;  // elements between rows of C (N, unless the launch covers a column range of a wider C)
+    int tiles_m, tiles_n;
+    long sa, sb, sc;  // batch strides in elements
+    // split-K (direct-to-LDS kernel only): blockIdx.z walks K tiles [z*kt_per_split, ...) and writes
+    // fp32 partial sums to partial[z][M][N]; a second kernel adds the splits in order.
+    int kt_per_split;
+    float* partial;
+    // One-launch split-K: one counter per C tile, zero between launches.  The workgroup that finishes a tile's last
+    // split adds the slabs in split order and writes C itself.  Null: a second kernel does that.
+    unsigned* tickets;
+    // K rotation: a workgroup walks its K tiles starting at (tile_n * rot_tile + xcd * rot_xcd) % KT and wraps.
+    // Workgroups that run at the same time then touch different column offsets of the 8 KB-strided rows, which
+    // spreads their requests over the memory channels (tile-shaped streaming of B from HBM: 4.3 -> 5.9 TB/s).
+    int rot_tile, rot_xcd;
+    // Tiles are numbered band by band: a band is band_m rows of tiles over all columns, walked column by column.
+    int band_m;
+    // Gated launches (kernels built with MODE 2): B holds two matrices `gate` rows apart, N counts the rows of both
+    // (2 x the output columns), and C[m][n] = silu(A[m,:].B[n,:]) * (A[m,:].B[gate + n,:]) for n < N / 2.
+    int gate;
+};
+
+// Map the linear workgroup id to a tile so that workgroups resident on one XCD (ids
+// congruent mod 8 are dispatched to the same XCD) work on neighbouring tiles: XCD x takes a contiguous run of
+// tile numbers, and tiles are numbered down a band of `band` rows of tiles, column after column, band after
+// band.  The 32 tiles an XCD works on at a time then cover about band x 32/band panels of A and B, which its
+// L2 serves to all of them; with more rows of tiles than `band` a whole column of tiles would share only its
+// panel of B and pull every panel of A through the L2 for a single use.
+__device__ __forceinline__ void tile_of_block(int bid, int nblocks, int tiles_m, int band, int& tm, int& tn) {
+    // nblocks / 8 tiles per XCD, one more on the first nblocks % 8 XCDs
+    const int x = bid & 7, base = nblocks >> 3, rem = nblocks & 7;
+    const int lid = x * base + (x < rem ? x : rem) + (bid >> 3);
+    if (band >= tiles_m) {
+        tm = lid % tiles_m;
+        tn = lid / tiles_m;
+        return;
+    }
+    const int tiles_n = nblocks / tiles_m;
+    const int per_band = band * tiles_n;
+    const int b = lid / per_band;
+    const int r = lid - b * per_band;
+    const int rows = (tiles_m - b * band) < band ? (tiles_m - b * band) : band;  // the last band may be lower
+    tm = b * band + r % rows;
+    tn = r / rows;
+}
+
+
+// The kernels of hgemm_vstage.hip (one wavefront per SIMD, K tiles in flight in registers).  band / rot_*: as in HgemmArgs.
+const char* hgemm_vstage_name(int index);
+bool hgemm_vstage_applies(const void* A, const void* B, const void* C, size_t M, size_t N, size_t K, size_t ldc);
+int launch_hgemm_vstage(int index, const void* A, const void* B, void* C, size_t M, size_t N, size_t K, size_t ldc, int band,
+                        int rot_tile, int rot_xcd);
+
+}  // namespace tl

@@ -648,3 +648,101 @@ def test_split_k_workspace_shared_by_two_host_threads(dev):
     finally:
         dev.lib.tl_set_hgemm_splits(0)
     assert not errors, errors[:3]
+
+
+# ---------------------------------------------------------------- split-K in one launch ----
+
+SPLIT_IN_LAUNCH_CASES = [
+    # (M, N, K), forced variant (None = dispatch), forced splits (0 = dispatch)
+    ((128, 4096, 4096), None, 0),
+    ((128, 4096, 11008), None, 0),
+    ((512, 4096, 4096), None, 2),                  # the dispatch covers this one with 256 unsplit tiles
+    ((512, 4096, 11008), None, 0),
+    ((128, 11008, 4096), None, 0),
+    ((130, 5128, 4096), None, 0),                  # partly filled last tiles in both directions
+    ((64, 8200, 8192), None, 0),
+    ((100, 1000, 1024), "p128x64x64w4x1s4", 3),    # splits that do not divide the K tiles evenly
+    ((300, 1096, 1472), "p128x128x64w2x4s4", 5),
+    ((512, 16640, 1024), "p128x256x64w2x4s3", 2),  # persistent kernel: 260 tiles on 256 workgroups, every tile ticketed
+    ((512, 16640, 512), "p256x128x64w2x4s3", 2),
+    ((256, 2048, 2048), "p128x128x64w2x2s4", 16),
+]
+
+
+@pytest.mark.parametrize("shape,variant,splits", SPLIT_IN_LAUNCH_CASES,
+                         ids=lambda v: "x".join(map(str, v)) if isinstance(v, tuple) else str(v))
+def test_hgemm_split_k_merged_inside_the_launch_equals_second_kernel(dev, oracle, shape, variant, splits):
+    """The workgroup that finishes a C tile's last split adds the fp32 slabs in split order and writes fp16 C itself
+    (per-tile tickets, device-coherent slabs; opt-in, the ordered second kernel is the faster default).  Same order, same
+    rounding: the two must agree bit for bit on random data, on every call of a sequence (the tickets return to
+    zero), and both must sit inside the gate against the oracle on sampled rows."""
+    M, N, K = shape
+    A = synth.normal_f16(8800 + M, (M, K), 1.0)
+    B = synth.normal_f16(8801 + N % 97, (N, K), 0.02)
+    Ad, Bd = dev.from_numpy(A), dev.from_numpy(B)
+    names = dev.hgemm_variants()
+    try:
+        if variant:
+            dev.set_hgemm_variant(names.index(variant))
+        dev.lib.tl_set_hgemm_splits(splits)
+        dev.lib.tl_set_hgemm_splitk_merge(2)
+        want = dev.hgemm(Ad, Bd).clone()
+        plan2 = dev.hgemm_last_plan()
+        assert dev.lib.tl_hgemm_last_split_in_launch() == 0
+        dev.lib.tl_set_hgemm_splitk_merge(1)
+        for rep in range(3):
+            got = dev.hgemm(Ad, Bd)
+            assert dev.hgemm_last_plan() == plan2
+            assert plan2[1] > 1, f"{shape}: the case is meant to split K, plan {plan2}"
+            assert dev.lib.tl_hgemm_last_split_in_launch() == 1
+            assert torch.equal(got, want), f"{shape} {plan2} call {rep}"
+        # a smaller problem right behind it reuses the same tickets and slabs
+        got2 = dev.hgemm(Ad[: max(2, M // 2)], Bd)
+        dev.lib.tl_set_hgemm_splitk_merge(2)
+        assert torch.equal(got2, dev.hgemm(Ad[: max(2, M // 2)], Bd))
+    finally:
+        dev.set_hgemm_variant(0)
+        dev.lib.tl_set_hgemm_splits(0)
+        dev.lib.tl_set_hgemm_splitk_merge(0)
+    rng = np.random.default_rng(M + N)
+    rows = np.unique(np.concatenate([[0, M - 1], rng.integers(0, M, 6)]))
+    assert_close_f16(want.cpu().numpy()[rows], oracle.matmul2d(A[rows], B), RTOL, ATOL, f"split-K {shape}")
+
+
+def test_hgemm_split_k_in_launch_integer_exact_and_reset(dev):
+    """Small integers are exact whatever the split; tl_reset_scratch() between calls leaves the tickets usable."""
+    for (M, N, K) in [(128, 4096, 4096), (96, 2048, 8192), (256, 4096, 11008)]:
+        A = synth.small_ints_f16(8900 + M, (M, K), -2, 2)
+        B = synth.small_ints_f16(8901 + N, (N, K), -1, 1)
+        Ad, Bd = dev.from_numpy(A), dev.from_numpy(B)
+        want = torch.from_numpy(A).cuda().double() @ torch.from_numpy(B).cuda().double().T
+        assert float(want.abs().max()) <= 2048
+        try:
+            dev.lib.tl_set_hgemm_splitk_merge(1)
+            for _ in range(2):
+                C = dev.hgemm(Ad, Bd)
+                assert dev.lib.tl_hgemm_last_split_in_launch() == 1, dev.hgemm_last_plan()
+                assert torch.equal(C.double(), want)
+                assert dev.lib.tl_reset_scratch() == 0
+        finally:
+            dev.lib.tl_set_hgemm_splitk_merge(0)
+        C = dev.hgemm(Ad, Bd)
+        assert dev.lib.tl_hgemm_last_split_in_launch() == 0 and torch.equal(C.double(), want)
+
+
+def test_hgemm_split_k_falls_back_to_the_second_kernel(dev):
+    """C rows that cannot take 8-byte stores (N % 8 != 0) keep the second kernel also when the in-launch merge is asked
+    for; the result is the same sum."""
+    M, N, K = 96, 1004, 4096
+    A = synth.small_ints_f16(8950, (M, K), -2, 2)
+    B = synth.small_ints_f16(8951, (N, K), -1, 1)
+    try:
+        dev.lib.tl_set_hgemm_splits(4)
+        dev.lib.tl_set_hgemm_splitk_merge(1)
+        C = dev.hgemm(dev.from_numpy(A), dev.from_numpy(B))
+        assert dev.hgemm_last_plan()[1] == 4 and dev.lib.tl_hgemm_last_split_in_launch() == 0
+    finally:
+        dev.lib.tl_set_hgemm_splits(0)
+        dev.lib.tl_set_hgemm_splitk_merge(0)
+    want = A.astype(np.float64) @ B.astype(np.float64).T
+    assert np.array_equal(C.cpu().numpy().astype(np.float64), want)
