@@ -777,9 +777,8 @@ static const HgemmVariant g_variants[] = {
     TL_HGEMM_PIPE(256, 192, 64, 2, 2, 2),  // 18
     // few rows: four wavefronts of 64x64 read a quarter fewer fragment bytes from LDS than eight of 64x32
     TL_HGEMM_PIPE(128, 128, 64, 2, 2, 4),  // 19
-    // hgemm_vstage.hip: one wavefront per SIMD, accumulators in AGPRs, two K tiles in flight in registers (stages < 0:
-    // index -stages - 1 into that file's table)
-    {"v256x256x64w2x2", 256, 256, 64, 256, -1, nullptr, true, nullptr},  // 20
+    // hgemm_big.hip: one wavefront per SIMD, 16x16x32 MFMAs, accumulators in AGPRs (stages < 0 marks it)
+    {"a256x256x64w2x2", 256, 256, 64, 256, -1, nullptr, true, nullptr},  // 20
 };
 
 static constexpr int kNumVariants = sizeof(g_variants) / sizeof(g_variants[0]);
@@ -1019,16 +1018,15 @@ static int launch_hgemm_cols(const void* A, const void* B, void* C, size_t M, si
         if (square_splits > 0) vi = v_square;
     }
     if (g_variants[vi].stages < 0) {
-        // the register-staged kernel: one dense fp16 C, no gate, no split; anything else falls back to the ring kernel
+        // whole 256x256 tiles of one dense fp16 C, no gate, no split; anything else falls back to the ring kernel
         const int forced_band = g_forced_band.load();
-        const int KTv = (int)(K / 64);
         const int rt = g_forced_rot_tile.load(), rx = g_forced_rot_xcd.load();
-        if (gate == 0 && batch == 1 && hgemm_vstage_applies(A, B, C, M, N, K, ldc)) {
+        if (gate == 0 && batch == 1 && hgemm_big_applies(A, B, C, M, N, K, ldc)) {
             g_last_variant = vi;
             g_last_splits = 1;
             g_last_one_launch = false;
-            return launch_hgemm_vstage(-g_variants[vi].stages - 1, A, B, C, M, N, K, ldc, forced_band > 0 ? forced_band : 8,
-                                       rt >= 0 ? rt : 0, rx >= 0 ? rx : KTv / 8);
+            return launch_hgemm_big(A, B, C, M, N, K, ldc, forced_band > 0 ? forced_band : 8, rt >= 0 ? rt : 0,
+                                    rx >= 0 ? rx : (int)(K / 64 / 8));
         }
         static const int v_big = hgemm_variant_index("p256x256x64w2x4s2");
         vi = v_big;

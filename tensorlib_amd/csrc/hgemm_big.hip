@@ -1,0 +1,346 @@
+// fp16 GEMM for many rows on 256x256 tiles, one wavefront per SIMD: C[M,N] = A[M,K] . B[N,K]^T, fp32 accumulation in the
+// MFMA accumulators, one rounding to fp16.  Same contract as the M > 1 branch of the reference's CUDA<half>::matmul2d
+// (tensorLib/src/device/cuda/gemm.cu:163-171 -> hgemm_cublas, tensorLib/src/device/cuda/hgemm.cu:20-38); numerics
+// follow CPU<half>::matmul2d (tensorLib/src/device/cpu/CPU.cpp:76-89).
+//
+// What it does differently from hgemm_f16_dlds_kernel (hgemm.hip), and why:
+//   * v_mfma_f32_16x16x32_f16 instead of 32x32x16.  The chip is power managed; out of registers, on operands that
+//     change with every instruction, the 16x16x32 shape sustains 1.80 PFLOP/s where 32x32x16 sustains 1.64 (it
+//     updates an accumulator half as often per flop), so the same schedule runs at a higher clock.
+//   * four wavefronts, one per SIMD, each owning a 128x128 piece of the tile: a third fewer fragment bytes read from
+//     LDS than eight wavefronts of 128x64.  That takes 256 accumulator registers per lane; they are pinned to the AGPR
+//     half of the register file by issuing the MFMA through inline assembly with an "a" constraint (left to itself
+//     the compiler keeps accumulators where the other values live, and spills), which leaves the VGPRs to fragments.
+//   * operand tiles go global -> LDS with global_load_lds_dwordx4 into a ring of two 64 KB stages, in the layout of the
+//     other kernel (a request is 8 rows x 128 bytes in lane order; the 16-byte chunk a lane fetches is permuted so that
+//     the fragment reads are free of bank conflicts).  A wavefront issues its 16 requests per K tile one every fourth
+//     MFMA (the CU's address path takes 16 cycles per request and four wavefronts share it), the first ones right
+//     behind the barrier that frees their stage.
+//   * the pipeline never drains between C tiles: a workgroup walks tiles blockIdx.x, + gridDim.x, ..., and the requests
+//     and fragment reads that run ahead of the MFMAs simply continue into the next C tile's first K tiles while the
+//     current tile's last MFMAs and its epilogue (staged through LDS behind the ring) are still under way.
+//   * the K loop is one straight chain of MFMAs per accumulator (every register array is indexed at compile time), so
+//     an accumulator never leaves the AGPR tuple it started in.
+// Both operands must come in whole tiles (M % 256 == 0, N % 256 == 0: the direct path has no bounds check) and K in an
+// even number of tiles of 64, at least four; the dispatch falls back to the other kernel otherwise.
+//
+// Measured on one MI355X (same box, W from HBM, random operands): 2048x32000x4096 412 us (1.30 PFLOP/s) against 470 us
+// for hgemm_f16_dlds_kernel<256,256,64,2,4,2,1>; 8192x8192x8192 768 against 844 us.  The same kernel with the tiles
+// travelling through registers (two K tiles in flight per wavefront, ds_write_b128 into the same ring) was built too,
+// for either operand or both: 433 us on the first shape.  A ds_write_b128 occupies the LDS pipeline five times as long
+// as a fragment read of the same size, which costs more than the deeper prefetch returns.
+#include <atomic>
+#include <type_traits>
+
+#include "hgemm_common.h"
+
+namespace tl {
+
+// f(integral_constant<int, I>) for I in [I0, N), expanded at compile time: every register array below is indexed with
+// constants, whatever the optimiser's unrolling limits are.
+template <int I, int N, typename F>
+__device__ __forceinline__ void static_for(F&& f) {
+    if constexpr (I < N) {
+        f(std::integral_constant<int, I>{});
+        static_for<I + 1, N>(f);
+    }
+}
+
+// acc += b-fragment . a-fragment with the accumulator in AGPRs.  B's fragment goes in as the first operand: the
+// accumulator then holds the tile transposed, lane l owning row (l % 16) of C and the four consecutive columns
+// 4 * (l / 16) .. + 3.
+__device__ __forceinline__ void mfma_agpr(float4_t& acc, const half8_t& b, const half8_t& a) {
+    asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(acc) : "v"(b), "v"(a));
+}
+
+// One global_load_lds_dwordx4: lane l's 16 bytes at base + offset[l] go to LDS bytes [lds_base + lds_imm + 16 l, + 16).
+template <int LDS_IMM>
+__device__ __forceinline__ void request_16B_per_lane(const void* uniform_base, unsigned lane_offset, unsigned lds_base) {
+    asm volatile("s_add_u32 m0, %2, %3\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %0"
+                 ::"s"(uniform_base), "v"(lane_offset), "s"(lds_base), "n"(LDS_IMM) : "memory", "scc");
+}
+
+// Idle cycles that every access to two rows of accumulators stays on its side of.  The MFMAs are hidden from the
+// compiler, so it neither knows that the matrix core may still be writing an accumulator the vector ALU is about to
+// read (up to 18 wait states) nor that a freshly written zero takes a few cycles to be readable by an MFMA: the
+// accumulators are operands of this statement, which orders it against every producer and consumer.
+#define TL_ACC_FENCE2(acc, i, text)                                                                                       \
+    asm volatile(text : "+a"(acc[i][0]), "+a"(acc[i][1]), "+a"(acc[i][2]), "+a"(acc[i][3]), "+a"(acc[i][4]),             \
+                 "+a"(acc[i][5]), "+a"(acc[i][6]), "+a"(acc[i][7]), "+a"(acc[i + 1][0]), "+a"(acc[i + 1][1]),              \
+                 "+a"(acc[i + 1][2]), "+a"(acc[i + 1][3]), "+a"(acc[i + 1][4]), "+a"(acc[i + 1][5]), "+a"(acc[i + 1][6]), \
+                 "+a"(acc[i + 1][7]))
+#define TL_ACC_FENCE(acc, text)       \
+    do {                              \
+        TL_ACC_FENCE2(acc, 0, text);  \
+        TL_ACC_FENCE2(acc, 2, "");    \
+        TL_ACC_FENCE2(acc, 4, "");    \
+        TL_ACC_FENCE2(acc, 6, "");    \
+    } while (0)
+
+// A_DIST: how many iterations (of NT MFMAs) ahead of its use an A fragment is read; D_STEP: MFMAs between two requests.
+template <int A_DIST, int D_STEP>
+__global__ void __launch_bounds__(256) hgemm_f16_big_kernel(HgemmArgs a) {
+    constexpr int BM = 256, BN = 256, BK = 64, WN = 2, NW = 4;
+    constexpr int RB = BK * 2;                 // bytes per tile row
+    constexpr int CPR = BK / 8;                // 16-byte chunks per tile row
+    constexpr int RPL = 256 / RB;              // tile rows per 256-byte LDS line
+    constexpr int RPW = 1024 / RB;             // tile rows written by one request
+    constexpr int A_REQS = BM / RPW / NW;      // requests per K tile, per wavefront and operand
+    constexpr int B_REQS = BN / RPW / NW;
+    constexpr int NREQ = A_REQS + B_REQS;
+    constexpr int A_BYTES = BM * RB;
+    constexpr int STAGE_BYTES = (BM + BN) * RB;
+    constexpr int TM = 128, TN = 128;          // wavefront tile
+    constexpr int MT = TM / 16, NT = TN / 16;  // 16x16 MFMA tiles per wavefront
+    constexpr int KS = BK / 32;                // K steps of 32 per K tile
+    constexpr int SLOTS = KS * MT * NT;        // MFMAs per K tile
+    constexpr int NA = KS * MT;                // A fragments per K tile
+    static_assert((NW * RPW / RPL) % CPR == 0, "the chunk a lane fetches must not depend on the request");
+    static_assert(A_REQS == B_REQS, "one set of lane offsets serves both operands");
+    // slot of the K tile's barrier: every read of the tile's own stage is issued before it, the first reads of the
+    // next tile's stage behind it
+    constexpr int BARRIER_SLOT = SLOTS - A_DIST * NT;
+    static_assert(NA % 4 == 0 && A_DIST >= 1 && A_DIST <= 3, "the A stream rotates through four registers");
+    static_assert(BARRIER_SLOT + NT < SLOTS, "the next tile's B fragments are read behind the barrier");
+    // request d < EARLY of K tile kt+2 goes out behind MFMA BARRIER_SLOT + 1 + D_STEP d of tile kt (the barrier has just
+    // freed its stage), the others behind MFMA 1 + D_STEP (d - EARLY) of tile kt+1
+    constexpr int EARLY_ROOM = (SLOTS - BARRIER_SLOT - 2) / D_STEP + 1;
+    constexpr int EARLY = EARLY_ROOM < NREQ ? EARLY_ROOM : NREQ;
+    constexpr int LATE = NREQ - EARLY;
+    static_assert(LATE == 0 || 1 + D_STEP * (LATE - 1) + 32 < BARRIER_SLOT, "a request needs time to land before its tile's barrier");
+
+    extern __shared__ __attribute__((aligned(1024))) unsigned char smem_raw[];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave / WN, wn = wave % WN;
+    const int N = a.N, K = a.K, ldc = a.ldc;
+    half_t* __restrict__ C = a.C;
+    const unsigned char* const Ag = reinterpret_cast<const unsigned char*>(a.A);
+    const unsigned char* const Bg = reinterpret_cast<const unsigned char*>(a.B);
+    const int KT = K / BK;              // even, at least 4 (host-checked)
+    const int total_tiles = a.tiles_m * a.tiles_n;
+    const int tiles_m = a.tiles_m, band_m = a.band_m;
+    const unsigned rot_tile = (unsigned)a.rot_tile, rot_xcd = (unsigned)a.rot_xcd;
+    const size_t row_bytes = (size_t)K * 2;
+
+    // Requests: request d of an operand covers, for this wavefront, tile rows (d * NW + wave) * RPW .. + RPW.  The
+    // lane's byte offset from the tile's first row at the K tile wanted is fixed for the whole kernel (one register
+    // per request, the same for both operands); the tile and the walk along K move a base pointer in scalar registers.
+    const int r0 = wave * RPW + lane / CPR;                       // tile row of request 0
+    const int chunk = (lane % CPR) ^ ((r0 / RPL) % CPR);           // the same for every request (static_assert above)
+    unsigned req_off[A_REQS];
+#pragma unroll
+    for (int d = 0; d < A_REQS; ++d) req_off[d] = (unsigned)(((size_t)(r0 + d * NW * RPW) * K + (size_t)chunk * 8) * 2);
+    const unsigned lds_wave = (unsigned)(unsigned long)(__attribute__((address_space(3))) unsigned char*)smem_raw + (unsigned)wave * 1024u;
+
+    // The request stream: the K tile whose requests come next, as base pointers into A and B, and where it sits in its
+    // C tile's walk (K tile k of the matrix, the w-th of the walk).  Past the last C tile the stream keeps asking for
+    // the last tile's data, which lands in stages nobody reads.
+    int req_vb = blockIdx.x, req_w = 0, req_k = 0;
+    const unsigned char *req_a_tile = Ag, *req_b_tile = Bg;     // first row of the C tile's panels
+    auto req_enter_tile = [&]() {
+        int tm, tn;
+        tile_of_block(req_vb, total_tiles, tiles_m, band_m, tm, tn);
+        req_a_tile = Ag + (size_t)tm * BM * row_bytes;
+        req_b_tile = Bg + (size_t)tn * BN * row_bytes;
+        req_w = 0;
+        req_k = (int)(((unsigned)tn * rot_tile + (blockIdx.x & 7u) * rot_xcd) % (unsigned)KT);
+    };
+    req_enter_tile();
+    const unsigned char *req_a = req_a_tile + (size_t)req_k * (BK * 2), *req_b = req_b_tile + (size_t)req_k * (BK * 2);
+    const unsigned char *late_a = req_a, *late_b = req_b;       // the K tile before it (its late requests are still due)
+    auto req_advance = [&]() {
+        late_a = req_a;
+        late_b = req_b;
+        ++req_w;
+        ++req_k;
+        if (req_k == KT) req_k = 0;
+        if (req_w == KT) {
+            if (req_vb + (int)gridDim.x < total_tiles) {
+                req_vb += (int)gridDim.x;
+                req_enter_tile();
+            } else {
+                req_w = 0;
+            }
+        }
+        req_a = req_a_tile + (size_t)req_k * (BK * 2);
+        req_b = req_b_tile + (size_t)req_k * (BK * 2);
+    };
+    // request d (A for d < A_REQS, else B) of the K tile at (pa, pb) into stage `stage` (a compile-time constant)
+    auto request = [&](auto dd, auto stage, const unsigned char* pa, const unsigned char* pb) {
+        constexpr int d = decltype(dd)::value, st = decltype(stage)::value;
+        if constexpr (d < A_REQS)
+            request_16B_per_lane<st * STAGE_BYTES + d * NW * 1024>(pa, req_off[d], lds_wave);
+        else
+            request_16B_per_lane<st * STAGE_BYTES + A_BYTES + (d - A_REQS) * NW * 1024>(pb, req_off[d - A_REQS], lds_wave);
+    };
+
+    // fragment reader: row (lane % 16) of a 16-row MFMA tile, chunk 4 * s + lane / 16 of K step s
+    const int fr_row = lane & 15;
+    const int fr_sw = (fr_row / RPL) % CPR;
+    int fr_off[KS];
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) fr_off[ks] = fr_row * RB + (((ks * 4 + (lane >> 4)) ^ fr_sw) * 16);
+    const unsigned char* const a_frag = smem_raw + wm * TM * RB;             // + stage, + 16-row block, + fr_off[s]
+    const unsigned char* const b_frag = smem_raw + A_BYTES + wn * TN * RB;
+
+    float4_t acc[MT][NT];
+    half8_t abuf[4];       // A fragment n of a K tile (n = s * MT + i) streams through abuf[n % 4]
+    half8_t bbuf[2][NT];   // the B fragments of K step s stay in bbuf[s] for the whole step
+    using S0 = std::integral_constant<int, 0>;
+    using S1 = std::integral_constant<int, 1>;
+    // This wavefront's requests have landed and its LDS reads are done, then the workgroup barrier.
+    auto tile_barrier = [&]() { asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory"); };
+
+    // prologue of the pipeline: K tile 0 of the first C tile into stage 0, the early requests of K tile 1 into stage 1
+    // (its late ones go out in the first slots of tile 0, as in every tile)
+    static_for<0, NREQ>([&](auto d) { request(d, S0{}, req_a, req_b); });
+    req_advance();
+    tile_barrier();
+    static_for<0, EARLY>([&](auto d) { request(d, S1{}, req_a, req_b); });
+    req_advance();
+    abuf[0] = *reinterpret_cast<const half8_t*>(a_frag + fr_off[0]);
+#pragma unroll
+    for (int j = 0; j < NT; ++j) bbuf[0][j] = *reinterpret_cast<const half8_t*>(b_frag + j * 16 * RB + fr_off[0]);
+#pragma unroll
+    for (int n = 1; n < A_DIST; ++n) abuf[n] = *reinterpret_cast<const half8_t*>(a_frag + n * 16 * RB + fr_off[0]);
+
+    // One K tile of the pipeline, the same for every tile of every C tile.  par: stage of this K tile (kt % 2).
+    // Slot q = (s * MT + i) * NT + j of the tile holds the MFMA of A fragment (s, i) and B fragment (s, j), and behind it:
+    //   j == 0: the read of A fragment n + A_DIST (from the next stage once n + A_DIST >= NA, i.e. behind the barrier);
+    //   step 0, j == 4: the read of B fragment i of step 1; the NT slots behind the barrier: the B fragments of the next tile;
+    //   slots 1 + D_STEP d': the late requests of K tile kt+1;  slots BARRIER_SLOT + 1 + D_STEP d: the early requests of
+    //   K tile kt+2, into the stage the barrier has just freed.
+    auto tile = [&](auto par) {
+        constexpr int P = decltype(par)::value;
+        using Cur = std::integral_constant<int, P>;
+        using Nxt = std::integral_constant<int, 1 - P>;
+        const unsigned char* const a_cur = a_frag + P * STAGE_BYTES;
+        const unsigned char* const b_cur = b_frag + P * STAGE_BYTES;
+        const unsigned char* const a_nxt = a_frag + (1 - P) * STAGE_BYTES;
+        const unsigned char* const b_nxt = b_frag + (1 - P) * STAGE_BYTES;
+        static_for<0, SLOTS>([&](auto slot) {
+            constexpr int q = decltype(slot)::value;
+            constexpr int s = q / (MT * NT), i = (q / NT) % MT, j = q % NT, n = s * MT + i;
+            if constexpr (q == BARRIER_SLOT) tile_barrier();   // tile kt+1 is complete in LDS, nobody reads tile kt's stage any more
+            mfma_agpr(acc[i][j], bbuf[s][j], abuf[n % 4]);
+            if constexpr (j == 0) {
+                constexpr int n2 = n + A_DIST;
+                if constexpr (n2 < NA)
+                    abuf[n2 % 4] = *reinterpret_cast<const half8_t*>(a_cur + (n2 % MT) * 16 * RB + fr_off[n2 / MT]);
+                else
+                    abuf[n2 % 4] = *reinterpret_cast<const half8_t*>(a_nxt + (n2 - NA) * 16 * RB + fr_off[0]);
+            }
+            if constexpr (s + 1 < KS && j == 4)
+                bbuf[(s + 1) % KS][i] = *reinterpret_cast<const half8_t*>(b_cur + i * 16 * RB + fr_off[(s + 1) % KS]);
+            if constexpr (q > BARRIER_SLOT && q - BARRIER_SLOT - 1 < NT)
+                bbuf[0][q - BARRIER_SLOT - 1] = *reinterpret_cast<const half8_t*>(b_nxt + (q - BARRIER_SLOT - 1) * 16 * RB + fr_off[0]);
+            if constexpr (q >= 1 && (q - 1) % D_STEP == 0 && (q - 1) / D_STEP < LATE)
+                request(std::integral_constant<int, EARLY + (q - 1) / D_STEP>{}, Nxt{}, late_a, late_b);
+            if constexpr (q > BARRIER_SLOT && (q - BARRIER_SLOT - 1) % D_STEP == 0 && (q - BARRIER_SLOT - 1) / D_STEP < EARLY)
+                request(std::integral_constant<int, (q - BARRIER_SLOT - 1) / D_STEP>{}, Cur{}, req_a, req_b);
+            __builtin_amdgcn_sched_barrier(0);
+        });
+        req_advance();
+    };
+
+    for (int vb = blockIdx.x;;) {   // C tiles of this workgroup
+#pragma unroll
+        for (int i = 0; i < MT; ++i)
+#pragma unroll
+            for (int j = 0; j < NT; ++j) acc[i][j] = float4_t{0.f, 0.f, 0.f, 0.f};
+        TL_ACC_FENCE(acc, "s_nop 7");
+
+        for (int kt = 0; kt < KT; kt += 2) {
+            tile(S0{});
+            tile(S1{});
+        }
+        TL_ACC_FENCE(acc, "s_nop 15\n\ts_nop 15");
+
+        // ---- epilogue.  acc[i][j][r] = C[row i*16 + lane%16][col j*16 + 4*(lane/16) + r] ----
+        // fp16 output through LDS: every wavefront turns 16 x TN blocks of its accumulators into row-major halves in a
+        // private region behind the ring (the ring itself already receives the next C tile's first K tiles), 8-byte
+        // writes into rows padded by 16 bytes, reads them back 16 bytes per lane and stores whole 16-byte pieces of C
+        // rows.  The host guarantees whole tiles, ldc % 8 == 0 and a 16-byte aligned C.
+        int tm, tn;
+        tile_of_block(vb, total_tiles, tiles_m, band_m, tm, tn);
+        const int e_row = lane & 15;
+        const int e_col = (lane >> 4) * 4;
+        const int row_base = tm * BM + wm * TM, col_base = tn * BN + wn * TN;
+        constexpr int RS = TN * 2 + 16;
+        constexpr int CH = TN / 8;               // 16-byte chunks per row
+        constexpr int RPR = 64 / CH;             // rows per wavefront-wide read
+        constexpr int PASSES = 16 / RPR;
+        static_assert(64 % CH == 0 && 16 % RPR == 0, "a staged block is read back in whole wavefront-wide passes");
+        unsigned char* region = smem_raw + 2 * STAGE_BYTES + wave * (16 * RS);
+#pragma unroll
+        for (int i = 0; i < MT; ++i) {
+#pragma unroll
+            for (int j = 0; j < NT; ++j) {
+                half4_t h = {(half_t)acc[i][j][0], (half_t)acc[i][j][1], (half_t)acc[i][j][2], (half_t)acc[i][j][3]};
+                *reinterpret_cast<half4_t*>(region + e_row * RS + (j * 16 + e_col) * 2) = h;
+            }
+#pragma unroll
+            for (int q = 0; q < PASSES; ++q) {
+                const int r = q * RPR + lane / CH, c = lane % CH;
+                const half8_t v = *reinterpret_cast<const half8_t*>(region + r * RS + c * 16);
+                const int row = row_base + i * 16 + r, col = col_base + c * 8;
+                if (col < N) *reinterpret_cast<half8_t*>(C + (size_t)row * ldc + col) = v;
+            }
+        }
+        vb += (int)gridDim.x;
+        if (vb >= total_tiles) break;
+    }
+    // requests that ran past the last tile may still be in flight towards LDS
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+}
+
+static std::atomic<bool> g_big_attr{false};
+
+const char* hgemm_big_name() { return "a256x256x64w2x2"; }
+
+// Full contract of the kernel: whole 256x256 tiles, an even number of K tiles of 64, at least four, lane offsets of a
+// tile within 32 bits, C rows that take 16-byte stores.
+bool hgemm_big_applies(const void* A, const void* B, const void* C, size_t M, size_t N, size_t K, size_t ldc) {
+    return M >= 256 && N >= 256 && M % 256 == 0 && N % 256 == 0 && K >= 256 && K % 128 == 0 && K <= ((size_t)1 << 22) &&
+           ldc % 8 == 0 && ldc >= N && aligned16(A) && aligned16(B) && aligned16(C) && M <= 0x7fffffffu && N <= 0x7fffffffu;
+}
+
+int launch_hgemm_big(const void* A, const void* B, void* C, size_t M, size_t N, size_t K, size_t ldc, int band, int rot_tile,
+                     int rot_xcd) {
+    TL_REQUIRE(hgemm_big_applies(A, B, C, M, N, K, ldc), "hgemm: %s does not serve this shape", hgemm_big_name());
+    void (*const kernel)(HgemmArgs) = hgemm_f16_big_kernel<2, 4>;
+    // the two-stage ring and behind it the C staging of the epilogue (four wavefronts x 16 rows x (256 + 16) bytes)
+    const size_t lds = (size_t)2 * (256 + 256) * 64 * sizeof(half_t) + (size_t)4 * 16 * (128 * 2 + 16);
+    if (!g_big_attr.load()) {
+        TL_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+        g_big_attr.store(true);
+    }
+    HgemmArgs a{};
+    a.A = (const half_t*)A;
+    a.B = (const half_t*)B;
+    a.C = (half_t*)C;
+    a.M = (int)M;
+    a.N = (int)N;
+    a.K = (int)K;
+    a.ldc = (int)ldc;
+    a.tiles_m = (int)(M / 256);
+    a.tiles_n = (int)(N / 256);
+    a.kt_per_split = 0x7fffffff;
+    a.band_m = band > 0 ? band : 8;
+    a.rot_tile = rot_tile;
+    a.rot_xcd = rot_xcd;
+    const size_t nblocks = (size_t)a.tiles_m * a.tiles_n;
+    TL_REQUIRE(nblocks <= 0x7fffffffu, "hgemm: too many tiles");
+    // persistent: one workgroup per CU walks tiles blockIdx.x, + gridDim.x, ...
+    size_t grid = nblocks;
+    const size_t cus = (size_t)device_info().cu_count;
+    if (cus > 0 && grid > cus) grid = cus;
+    hipLaunchKernelGGL(kernel, dim3((unsigned)grid), dim3(256), lds, stream(), a);
+    TL_CHECK_LAUNCH(hgemm_big_name());
+    return TL_OK;
+}
+
+}  // namespace tl

@@ -56,10 +56,11 @@ __device__ __forceinline__ void tile_of_block(int bid, int nblocks, int tiles_m,
 }
 
 
-// The kernels of hgemm_vstage.hip (one wavefront per SIMD, K tiles in flight in registers).  band / rot_*: as in HgemmArgs.
-const char* hgemm_vstage_name(int index);
-bool hgemm_vstage_applies(const void* A, const void* B, const void* C, size_t M, size_t N, size_t K, size_t ldc);
-int launch_hgemm_vstage(int index, const void* A, const void* B, void* C, size_t M, size_t N, size_t K, size_t ldc, int band,
-                        int rot_tile, int rot_xcd);
+// The kernel of hgemm_big.hip (256x256 tiles, one wavefront per SIMD, accumulators in AGPRs).  band / rot_*: as in
+// HgemmArgs.
+const char* hgemm_big_name();
+bool hgemm_big_applies(const void* A, const void* B, const void* C, size_t M, size_t N, size_t K, size_t ldc);
+int launch_hgemm_big(const void* A, const void* B, void* C, size_t M, size_t N, size_t K, size_t ldc, int band, int rot_tile,
+                     int rot_xcd);
 
 }  // namespace tl
