@@ -826,7 +826,9 @@ static bool hgemm_many_rows_split(size_t M, size_t N, size_t K, int cus) {
     return M > 512 && K >= 8192 && t * 2 <= (size_t)cus && t * 22016 <= (size_t)cus * K;
 }
 
-static HgemmPlan plan_many_rows(size_t M, size_t N, size_t K, int cus, bool can_split) {
+// fast_big: the problem comes in whole 256x256 tiles that hgemm_big.hip's kernel can take (a round of them then costs
+// 0.87 of a round of the ring kernel's: 2048x32000x4096 405 against 475 us on one box)
+static HgemmPlan plan_many_rows(size_t M, size_t N, size_t K, int cus, bool can_split, bool fast_big = false) {
     static const int v_big = hgemm_variant_index("p256x256x64w2x4s2");
     static const int v_mid = hgemm_variant_index("p128x256x64w2x4s3");
     static const int v_small = hgemm_variant_index("p128x128x64w2x4s2");
@@ -846,7 +848,7 @@ static HgemmPlan plan_many_rows(size_t M, size_t N, size_t K, int cus, bool can_
         if (can_split && hgemm_many_rows_split(M, N, K, cus)) return {v_mid, c_small};
         return {v_few_128x128, c_small};
     }
-    const double c_big = cost(tiles(256, 256), (size_t)cus, 1.0);
+    const double c_big = cost(tiles(256, 256), (size_t)cus, fast_big ? 0.87 : 1.0);
     const double c_mid = cost(tiles(128, 256), (size_t)cus, 0.613);
     const double c_192 = cost(tiles(256, 192), (size_t)cus, 0.865);   // three quarters of the work at 0.865 of the cost
     int best = v_big;
@@ -897,7 +899,7 @@ static int square_tile_splits(size_t M, size_t N, size_t K, int cus, bool can_sp
     return sp;
 }
 
-static int pick_variant(size_t M, size_t N, size_t K, int cus, bool can_split) {
+static int pick_variant(size_t M, size_t N, size_t K, int cus, bool can_split, bool fast_big = false) {
     static const int v_big = hgemm_variant_index("p256x256x64w2x4s2");
     static const int v_mid = hgemm_variant_index("p128x256x64w2x4s3");
     static const int v_few_256x128 = hgemm_variant_index("p256x128x64w2x4s3");
@@ -928,7 +930,7 @@ static int pick_variant(size_t M, size_t N, size_t K, int cus, bool can_split) {
         if (tiles(128, 64) > (size_t)cus) return v_few_128x128;
         return v_few_128x64;
     }
-    return plan_many_rows(M, N, K, cus, can_split).variant;
+    return plan_many_rows(M, N, K, cus, can_split, fast_big).variant;
 }
 
 // One launch (plus the ordered reduce when K is split) for columns [0, N) of a C whose rows are ldc elements apart.
@@ -955,11 +957,14 @@ int launch_hgemm(const void* A, const void* B, void* C, size_t M, size_t N, size
             const size_t full = col_tiles / cols_per_round, rem = col_tiles % cols_per_round;
             if (full >= 1 && rem > 0) {
                 const size_t N1 = full * cols_per_round * 256;
-                const double whole = plan_many_rows(M, N, K, cus, true).cost;
-                const double split = (double)full * (double)(tiles_m * cols_per_round) / (double)cus +
-                                     plan_many_rows(M, N - N1, K, cus, false).cost + 0.04;   // 0.04: the second launch's ramp
+                const size_t c1 = gate ? N1 / 2 : N1;   // first column of C (and row of B) of the second launch
+                const bool fast_all = gate == 0 && hgemm_big_applies(A, B, C, M, N, K, ldc_all);
+                const bool fast_first = gate == 0 && hgemm_big_applies(A, B, C, M, N1, K, ldc_all);
+                const bool fast_rest = gate == 0 && hgemm_big_applies(A, (const half_t*)B + c1 * K, (half_t*)C + c1, M, N - N1, K, ldc_all);
+                const double whole = plan_many_rows(M, N, K, cus, true, fast_all).cost;
+                const double split = (fast_first ? 0.87 : 1.0) * (double)full * (double)(tiles_m * cols_per_round) / (double)cus +
+                                     plan_many_rows(M, N - N1, K, cus, false, fast_rest).cost + 0.04;   // 0.04: the second launch's ramp
                 if (split < whole * 0.97) {
-                    const size_t c1 = gate ? N1 / 2 : N1;   // first column of C (and row of B) of the second launch
                     int rc = launch_hgemm_cols(A, B, C, M, N1, K, ldc_all, 1, 0, 0, 0, nullptr, nullptr, nullptr, v_big, gate);
                     if (rc != TL_OK) return rc;
                     if (splits_out) *splits_out = 1;
@@ -1010,7 +1015,14 @@ static int launch_hgemm_cols(const void* A, const void* B, void* C, size_t M, si
         return launch_hgemm_fewrows(A, B, C, M, N, K, ldc);
     }
     const bool can_split = batch == 1 && ldc == N;   // the second pass of a split K writes a dense C
-    int vi = forced_variant ? forced_variant : pick_variant(M, N, K, device_info().cu_count, can_split);
+    // whole 256x256 tiles of a single dense C: where the 256x256 ring kernel would run, hgemm_big.hip's kernel does
+    const bool fast_big = gate == 0 && batch == 1 && g_forced_variant.load() == 0 && hgemm_big_applies(A, B, C, M, N, K, ldc);
+    int vi = forced_variant ? forced_variant : pick_variant(M, N, K, device_info().cu_count, can_split, fast_big);
+    {
+        static const int v_big = hgemm_variant_index("p256x256x64w2x4s2");
+        static const int v_fast = hgemm_variant_index("a256x256x64w2x2");
+        if (fast_big && vi == v_big) vi = v_fast;
+    }
     int square_splits = 0;
     if (forced_variant == 0 && g_forced_splits.load() == 0) {
         square_splits = square_tile_splits(M, N, K, device_info().cu_count, can_split);

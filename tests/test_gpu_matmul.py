@@ -403,6 +403,20 @@ def test_hgemm_silu_mul_equals_two_steps(dev, shape):
     assert_close_f16(got.cpu().numpy(), ref.cpu().numpy().astype(np.float16), RTOL, 2e-3, f"gated {shape}")
 
 
+@pytest.mark.parametrize("M", [128, 512, 2048])
+def test_hgemm_silu_mul_against_the_oracle(dev, oracle, M):
+    """The gated w1|w3 projection against the CPU restatement directly, on eight sampled rows at the Llama2-7B size:
+    oracle.silu_mul(oracle.matmul2d(X, W1), oracle.matmul2d(X, W3)) at the gate of the single kernels."""
+    hidden, K = 11008, 4096
+    X = synth.normal_f16(7850 + M, (M, K), 1.0)
+    W13 = synth.normal_f16(7851, (2 * hidden, K), 0.02)
+    got = dev.hgemm_silu_mul(dev.from_numpy(X), dev.from_numpy(W13)).cpu().numpy()
+    rng = np.random.default_rng(M)
+    rows = np.unique(np.concatenate([[0, M - 1], rng.integers(0, M, 6)]))
+    want = oracle.silu_mul(oracle.matmul2d(X[rows], W13[:hidden]), oracle.matmul2d(X[rows], W13[hidden:]))
+    assert_close_f16(got[rows], want, RTOL, ATOL, f"gated {M}x{hidden}x{K} against the oracle")
+
+
 def test_hgemm_silu_mul_drawn_shapes(dev):
     """Forty drawn shapes (rows 2..700, hidden a multiple of 8 up to 3000, K a multiple of 64 up to 2048) through the
     automatic dispatch: tiles partly filled in both directions, column ranges, every tile shape the dispatch reaches."""
@@ -746,3 +760,84 @@ def test_hgemm_split_k_falls_back_to_the_second_kernel(dev):
         dev.lib.tl_set_hgemm_splitk_merge(0)
     want = A.astype(np.float64) @ B.astype(np.float64).T
     assert np.array_equal(C.cpu().numpy().astype(np.float64), want)
+
+
+# ------------------------------------------------------- the dispatch of the benchmark shapes ----
+
+BASELINE_PLANS = [
+    # (M, N, K), (variant of the last launch, K splits): the twelve prefill shapes and the four projections of a 16-token
+    # prompt on a 256-CU MI355X
+    ((2048, 4096, 4096), ("p128x256x64w2x4s3", 1)),
+    ((2048, 11008, 4096), ("p128x256x64w2x4s3", 1)),   # 8192 columns of 256x256 tiles first, this is the launch for the rest
+    ((2048, 32000, 4096), ("a256x256x64w2x2", 1)),
+    ((2048, 4096, 11008), ("p128x256x64w2x4s3", 1)),
+    ((512, 4096, 4096), ("p128x64x64w4x1s4", 1)),
+    ((512, 11008, 4096), ("p128x192x64w4x2s4", 1)),
+    ((512, 32000, 4096), ("a256x256x64w2x2", 1)),
+    ((512, 4096, 11008), ("p128x256x64w2x4s3", 4)),
+    ((128, 4096, 4096), ("p128x64x64w4x1s4", 4)),
+    ((128, 11008, 4096), ("p128x128x64w2x2s4", 2)),
+    ((128, 32000, 4096), ("p128x128x64w2x2s4", 1)),
+    ((128, 4096, 11008), ("p128x64x64w4x1s4", 4)),
+    ((16, 12288, 4096), ("fewrows", 1)),
+    ((16, 4096, 4096), ("fewrows", 1)),
+    ((16, 22016, 4096), ("fewrows", 1)),
+    ((16, 4096, 11008), ("p128x64x64w4x1s4", 4)),
+]
+
+
+@pytest.mark.parametrize("shape,plan", BASELINE_PLANS, ids=lambda v: "x".join(map(str, v)) if isinstance(v[0], int) else None)
+def test_hgemm_dispatch_of_the_benchmark_shapes_is_pinned(dev, shape, plan):
+    """The kernel variant and the K split the dispatch takes for every shape bench.py reports (the plans were measured
+    on a 256-CU MI355X; a retune that moves one of them has to change this table and re-measure the shape)."""
+    if dev.lib.tl_device_cu_count() != 256:
+        pytest.skip("plans are pinned for 256 compute units")
+    M, N, K = shape
+    A = dev.from_numpy(synth.small_ints_f16(9100 + M, (M, K), -1, 1))
+    B = dev.from_numpy(synth.small_ints_f16(9101 + N % 89, (N, K), -1, 1))
+    C = dev.hgemm(A, B)
+    assert dev.hgemm_last_plan() == plan
+    rows = [0, M // 2, M - 1]
+    want = A[rows].double() @ B.double().T
+    assert float(want.abs().max()) <= 2048 and torch.equal(C[rows].double(), want)
+
+
+@pytest.mark.parametrize("shape", [(256, 256, 256), (512, 768, 384), (2048, 40960, 512), (2560, 11008, 1024), (1024, 1024, 11008)],
+                         ids=lambda s: "x".join(map(str, s)))
+def test_hgemm_256x256_agpr_kernel_integer_exact(dev, shape):
+    """hgemm_f16_big_kernel forced on whole-tile shapes: one tile, fewer tiles than compute units, several tiles per
+    workgroup (the pipeline runs on into the next C tile), K walks rotated per tile and per XCD.  Small integers are
+    exact whatever the order of the fp32 sums, so a K tile skipped, repeated or taken from the wrong C tile shows as a
+    wrong bit."""
+    M, N, K = shape
+    A = dev.from_numpy(synth.small_ints_f16(9200 + M, (M, K), -2, 2))
+    B = dev.from_numpy(synth.small_ints_f16(9201 + N % 83, (N, K), -2, 2))
+    want = A.double() @ B.double().T
+    assert float(want.abs().max()) <= 2048
+    V = dev.hgemm_variants().index("a256x256x64w2x2")
+    try:
+        dev.set_hgemm_variant(V)
+        for rot in ((-1, -1), (0, 0), (3, 5), (1000003, 17)):
+            dev.lib.tl_set_hgemm_k_rotation(*rot)
+            C = dev.hgemm(A, B)
+            assert dev.hgemm_last_plan() == ("a256x256x64w2x2", 1)
+            assert torch.equal(C.double(), want), (shape, rot)
+    finally:
+        dev.set_hgemm_variant(0)
+        dev.lib.tl_set_hgemm_k_rotation(-1, -1)
+
+
+def test_hgemm_256x256_agpr_kernel_falls_back_on_partial_tiles(dev, oracle):
+    """Rows or columns that do not fill whole 256x256 tiles, a K that is not an even number of tiles: the forced variant
+    hands the call to the ring kernel."""
+    V = dev.hgemm_variants().index("a256x256x64w2x2")
+    try:
+        dev.set_hgemm_variant(V)
+        for (M, N, K) in [(300, 512, 256), (512, 520, 256), (512, 512, 192), (256, 256, 128)]:
+            A = synth.small_ints_f16(9300 + M, (M, K), -2, 2)
+            B = synth.small_ints_f16(9301 + N, (N, K), -2, 2)
+            C = dev.hgemm(dev.from_numpy(A), dev.from_numpy(B)).cpu().numpy()
+            assert dev.hgemm_last_plan()[0] != "a256x256x64w2x2"
+            assert np.array_equal(C.view(np.uint16), oracle.matmul2d(A, B).view(np.uint16)), (M, N, K)
+    finally:
+        dev.set_hgemm_variant(0)

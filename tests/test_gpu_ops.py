@@ -380,6 +380,35 @@ def test_hgemm_prefill_rope_qkv_vt_equals_separate_calls(dev, S, H, D, K):
     assert torch.equal(q2, q1) and torch.equal(k2, k1) and torch.equal(v2, v1) and torch.equal(vT2, vT1), f"splits {split}"
 
 
+@pytest.mark.parametrize("S", [128, 512, 33])
+def test_hgemm_prefill_rope_qkv_vt_against_the_oracle(dev, oracle, S):
+    """The fused projection + rotation entry against the CPU restatement directly: oracle.matmul2d of sampled token rows
+    through wq, wk and wv, oracle.rope of the q and k rows at the tokens' positions.  The projection differs from the
+    oracle's only in the order of the fp32 sum (gate of the GEMM tests); the rotation then acts on those fp16 values,
+    so the rotated outputs are gated the same way and the v rows must equal the GEMM's own output bit for bit."""
+    H, D, K = 32, 128, 4096
+    dim = H * D
+    X = synth.normal_f16(190 + S, (S, K), 1.0)
+    W = synth.normal_f16(191 + S, (3 * dim, K), 0.02)
+    Xd, Wd = dev.from_numpy(X), dev.from_numpy(W)
+    table = dev.rope_table(max(S, 8), D)
+    kc, vc = dev.empty(S, H, D), dev.empty(S, H, D)
+    q, vT = dev.hgemm_prefill_rope_qkv_vt(Xd, Wd, kc, vc, table, H)            # q [H, S, D], vT [H, D, ldv]
+    rng = np.random.default_rng(S)
+    rows = np.unique(np.concatenate([[0, S - 1], rng.integers(0, S, 6)]))
+    qkv = oracle.matmul2d(X[rows], W)                                           # [rows, 3 dim]
+    qn, kn, vn, vTn = q.cpu().numpy(), kc.cpu().numpy(), vc.cpu().numpy(), vT.cpu().numpy()
+    for i, t in enumerate(rows):
+        want_q = oracle.rope(qkv[i, :dim].reshape(1, 1, H, D), int(t))[0, 0]
+        want_k = oracle.rope(qkv[i, dim:2 * dim].reshape(1, 1, H, D), int(t))[0, 0]
+        want_v = qkv[i, 2 * dim:].reshape(H, D)
+        # a rotated value mixes two products of size |x|: gate on the pair's magnitude like the chain tests gate on rms
+        assert_close_f16(qn[:, t, :], want_q, RTOL, 2 * ATOL, f"fused q row {t}")
+        assert_close_f16(kn[t], want_k, RTOL, 2 * ATOL, f"fused k row {t}")
+        assert_close_f16(vn[t], want_v, RTOL, ATOL, f"fused v row {t}")
+        assert np.array_equal(vTn[:, :, t].view(np.uint16), vn[t].view(np.uint16))
+
+
 @pytest.mark.parametrize("D", [64, 128])
 @pytest.mark.parametrize("chunk", [64, 128, 256])
 def test_decode_attention_every_chunk_size_vs_chain(dev, oracle, chunk, D):
