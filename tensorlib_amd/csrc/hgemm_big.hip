@@ -52,6 +52,11 @@ __device__ __forceinline__ void static_for(F&& f) {
 __device__ __forceinline__ void mfma_agpr(float4_t& acc, const half8_t& b, const half8_t& a) {
     asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(acc) : "v"(b), "v"(a));
 }
+// acc = b-fragment . a-fragment: the first MFMA of a C tile starts the accumulator from the constant zero, so the
+// 256 accumulator registers are never cleared by the vector ALU.
+__device__ __forceinline__ void mfma_agpr_first(float4_t& acc, const half8_t& b, const half8_t& a) {
+    asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, 0" : "=a"(acc) : "v"(b), "v"(a));
+}
 
 // One global_load_lds_dwordx4: lane l's 16 bytes at base + offset[l] go to LDS bytes [lds_base + lds_imm + 16 l, + 16).
 template <int LDS_IMM>
@@ -77,8 +82,9 @@ __device__ __forceinline__ void request_16B_per_lane(const void* uniform_base, u
         TL_ACC_FENCE2(acc, 6, "");    \
     } while (0)
 
-// A_DIST: how many iterations (of NT MFMAs) ahead of its use an A fragment is read; D_STEP: MFMAs between two requests.
-template <int A_DIST, int D_STEP>
+// A_AHEAD: how many iterations (of NT MFMAs) ahead of its use an A fragment is read; BAR_IT: the iteration in front of
+// which the K tile's barrier stands; D_STEP: MFMAs between two requests.
+template <int A_AHEAD, int BAR_IT, int D_STEP>
 __global__ void __launch_bounds__(256) hgemm_f16_big_kernel(HgemmArgs a) {
     constexpr int BM = 256, BN = 256, BK = 64, WN = 2, NW = 4;
     constexpr int RB = BK * 2;                 // bytes per tile row
@@ -97,17 +103,20 @@ __global__ void __launch_bounds__(256) hgemm_f16_big_kernel(HgemmArgs a) {
     constexpr int NA = KS * MT;                // A fragments per K tile
     static_assert((NW * RPW / RPL) % CPR == 0, "the chunk a lane fetches must not depend on the request");
     static_assert(A_REQS == B_REQS, "one set of lane offsets serves both operands");
-    // slot of the K tile's barrier: every read of the tile's own stage is issued before it, the first reads of the
-    // next tile's stage behind it
-    constexpr int BARRIER_SLOT = SLOTS - A_DIST * NT;
-    static_assert(NA % 4 == 0 && A_DIST >= 1 && A_DIST <= 3, "the A stream rotates through four registers");
-    static_assert(BARRIER_SLOT + NT < SLOTS, "the next tile's B fragments are read behind the barrier");
+    // Slot of the K tile's barrier.  Every read of the tile's own stage is issued before it (A fragment n at iteration
+    // n - A_AHEAD, the B fragments of step 1 during step 0), early enough that the data has arrived when the barrier
+    // is reached; the first reads of the next tile's stage (its first A_AHEAD A fragments and the B fragments of its
+    // step 0) stand behind it.
+    constexpr int BARRIER_SLOT = BAR_IT * NT;
+    static_assert(A_AHEAD >= 1 && NA - 1 - A_AHEAD < BAR_IT && BAR_IT < NA, "the last A fragment is requested before the barrier");
+    static_assert(BARRIER_SLOT + 2 * (NT + A_AHEAD) <= SLOTS, "the next tile's first fragments are read behind the barrier");
     // request d < EARLY of K tile kt+2 goes out behind MFMA BARRIER_SLOT + 1 + D_STEP d of tile kt (the barrier has just
     // freed its stage), the others behind MFMA 1 + D_STEP (d - EARLY) of tile kt+1
     constexpr int EARLY_ROOM = (SLOTS - BARRIER_SLOT - 2) / D_STEP + 1;
     constexpr int EARLY = EARLY_ROOM < NREQ ? EARLY_ROOM : NREQ;
     constexpr int LATE = NREQ - EARLY;
     static_assert(LATE == 0 || 1 + D_STEP * (LATE - 1) + 32 < BARRIER_SLOT, "a request needs time to land before its tile's barrier");
+    static_assert(NA % 4 == 0, "fragment counts");
 
     extern __shared__ __attribute__((aligned(1024))) unsigned char smem_raw[];
 
@@ -187,7 +196,7 @@ __global__ void __launch_bounds__(256) hgemm_f16_big_kernel(HgemmArgs a) {
     const unsigned char* const b_frag = smem_raw + A_BYTES + wn * TN * RB;
 
     float4_t acc[MT][NT];
-    half8_t abuf[4];       // A fragment n of a K tile (n = s * MT + i) streams through abuf[n % 4]
+    half8_t abuf[NA];      // A fragment n of a K tile (n = s * MT + i)
     half8_t bbuf[2][NT];   // the B fragments of K step s stay in bbuf[s] for the whole step
     using S0 = std::integral_constant<int, 0>;
     using S1 = std::integral_constant<int, 1>;
@@ -205,16 +214,19 @@ __global__ void __launch_bounds__(256) hgemm_f16_big_kernel(HgemmArgs a) {
 #pragma unroll
     for (int j = 0; j < NT; ++j) bbuf[0][j] = *reinterpret_cast<const half8_t*>(b_frag + j * 16 * RB + fr_off[0]);
 #pragma unroll
-    for (int n = 1; n < A_DIST; ++n) abuf[n] = *reinterpret_cast<const half8_t*>(a_frag + n * 16 * RB + fr_off[0]);
+    for (int n = 1; n < A_AHEAD; ++n) abuf[n] = *reinterpret_cast<const half8_t*>(a_frag + n * 16 * RB + fr_off[0]);
 
     // One K tile of the pipeline, the same for every tile of every C tile.  par: stage of this K tile (kt % 2).
     // Slot q = (s * MT + i) * NT + j of the tile holds the MFMA of A fragment (s, i) and B fragment (s, j), and behind it:
-    //   j == 0: the read of A fragment n + A_DIST (from the next stage once n + A_DIST >= NA, i.e. behind the barrier);
-    //   step 0, j == 4: the read of B fragment i of step 1; the NT slots behind the barrier: the B fragments of the next tile;
+    //   j == 0: the read of A fragment n + A_AHEAD of this tile;  step 0, j == 4: the read of B fragment i of step 1;
+    //   behind the barrier, every second slot: A fragment 0, the B fragments of step 0 and A fragments 1 .. A_AHEAD - 1 of
+    //   the next tile, in the order its MFMAs need them;
     //   slots 1 + D_STEP d': the late requests of K tile kt+1;  slots BARRIER_SLOT + 1 + D_STEP d: the early requests of
     //   K tile kt+2, into the stage the barrier has just freed.
-    auto tile = [&](auto par) {
+    // first: the K tile opens a C tile (its first K step starts the accumulators from zero)
+    auto tile = [&](auto par, auto first) {
         constexpr int P = decltype(par)::value;
+        constexpr bool FIRST = decltype(first)::value;
         using Cur = std::integral_constant<int, P>;
         using Nxt = std::integral_constant<int, 1 - P>;
         const unsigned char* const a_cur = a_frag + P * STAGE_BYTES;
@@ -225,18 +237,21 @@ __global__ void __launch_bounds__(256) hgemm_f16_big_kernel(HgemmArgs a) {
             constexpr int q = decltype(slot)::value;
             constexpr int s = q / (MT * NT), i = (q / NT) % MT, j = q % NT, n = s * MT + i;
             if constexpr (q == BARRIER_SLOT) tile_barrier();   // tile kt+1 is complete in LDS, nobody reads tile kt's stage any more
-            mfma_agpr(acc[i][j], bbuf[s][j], abuf[n % 4]);
-            if constexpr (j == 0) {
-                constexpr int n2 = n + A_DIST;
-                if constexpr (n2 < NA)
-                    abuf[n2 % 4] = *reinterpret_cast<const half8_t*>(a_cur + (n2 % MT) * 16 * RB + fr_off[n2 / MT]);
-                else
-                    abuf[n2 % 4] = *reinterpret_cast<const half8_t*>(a_nxt + (n2 - NA) * 16 * RB + fr_off[0]);
+            if constexpr (FIRST && s == 0) mfma_agpr_first(acc[i][j], bbuf[s][j], abuf[n]);
+            else mfma_agpr(acc[i][j], bbuf[s][j], abuf[n]);
+            if constexpr (j == 0 && n + A_AHEAD < NA) {
+                constexpr int n2 = n + A_AHEAD;
+                abuf[n2] = *reinterpret_cast<const half8_t*>(a_cur + (n2 % MT) * 16 * RB + fr_off[n2 / MT]);
             }
             if constexpr (s + 1 < KS && j == 4)
                 bbuf[(s + 1) % KS][i] = *reinterpret_cast<const half8_t*>(b_cur + i * 16 * RB + fr_off[(s + 1) % KS]);
-            if constexpr (q > BARRIER_SLOT && q - BARRIER_SLOT - 1 < NT)
-                bbuf[0][q - BARRIER_SLOT - 1] = *reinterpret_cast<const half8_t*>(b_nxt + (q - BARRIER_SLOT - 1) * 16 * RB + fr_off[0]);
+            // r-th read behind the barrier: A0, B0 .. B(NT-1), A1 ..
+            if constexpr (q > BARRIER_SLOT && (q - BARRIER_SLOT - 1) % 2 == 0 && (q - BARRIER_SLOT - 1) / 2 < NT + A_AHEAD) {
+                constexpr int r = (q - BARRIER_SLOT - 1) / 2;
+                if constexpr (r == 0) abuf[0] = *reinterpret_cast<const half8_t*>(a_nxt + fr_off[0]);
+                else if constexpr (r <= NT) bbuf[0][r - 1] = *reinterpret_cast<const half8_t*>(b_nxt + (r - 1) * 16 * RB + fr_off[0]);
+                else abuf[r - NT] = *reinterpret_cast<const half8_t*>(a_nxt + (r - NT) * 16 * RB + fr_off[0]);
+            }
             if constexpr (q >= 1 && (q - 1) % D_STEP == 0 && (q - 1) / D_STEP < LATE)
                 request(std::integral_constant<int, EARLY + (q - 1) / D_STEP>{}, Nxt{}, late_a, late_b);
             if constexpr (q > BARRIER_SLOT && (q - BARRIER_SLOT - 1) % D_STEP == 0 && (q - BARRIER_SLOT - 1) / D_STEP < EARLY)
@@ -247,15 +262,11 @@ __global__ void __launch_bounds__(256) hgemm_f16_big_kernel(HgemmArgs a) {
     };
 
     for (int vb = blockIdx.x;;) {   // C tiles of this workgroup
-#pragma unroll
-        for (int i = 0; i < MT; ++i)
-#pragma unroll
-            for (int j = 0; j < NT; ++j) acc[i][j] = float4_t{0.f, 0.f, 0.f, 0.f};
-        TL_ACC_FENCE(acc, "s_nop 7");
-
-        for (int kt = 0; kt < KT; kt += 2) {
-            tile(S0{});
-            tile(S1{});
+        tile(S0{}, std::true_type{});
+        tile(S1{}, std::false_type{});
+        for (int kt = 2; kt < KT; kt += 2) {
+            tile(S0{}, std::false_type{});
+            tile(S1{}, std::false_type{});
         }
         TL_ACC_FENCE(acc, "s_nop 15\n\ts_nop 15");
 
@@ -311,7 +322,9 @@ bool hgemm_big_applies(const void* A, const void* B, const void* C, size_t M, si
 int launch_hgemm_big(const void* A, const void* B, void* C, size_t M, size_t N, size_t K, size_t ldc, int band, int rot_tile,
                      int rot_xcd) {
     TL_REQUIRE(hgemm_big_applies(A, B, C, M, N, K, ldc), "hgemm: %s does not serve this shape", hgemm_big_name());
-    void (*const kernel)(HgemmArgs) = hgemm_f16_big_kernel<2, 4>;
+    // A fragments read three iterations ahead, the barrier in front of iteration 13 of 16, a request every fourth MFMA:
+    // A_AHEAD 3 .. 6, barriers at 11 .. 13 and request spacings 3 and 4 measured within 1 % of each other
+    void (*const kernel)(HgemmArgs) = hgemm_f16_big_kernel<3, 13, 4>;
     // the two-stage ring and behind it the C staging of the epilogue (four wavefronts x 16 rows x (256 + 16) bytes)
     const size_t lds = (size_t)2 * (256 + 256) * 64 * sizeof(half_t) + (size_t)4 * 16 * (128 * 2 + 16);
     if (!g_big_attr.load()) {
