@@ -135,6 +135,10 @@ int tl_set_hgemm_splits(int splits);
 /* Inspection hook (no reference counterpart): the kernel variant (index into tl_hgemm_variant_name(); -1 = the
  * kernel for at most 32 rows) and the number of K splits the most recent fp16 GEMM launch of this process used. */
 int tl_hgemm_last_plan(int* variant, int* splits);
+/* Tuning hook: 0 = the dispatch takes the kernels with 16x16x32 MFMAs and accumulators in AGPRs (variants
+ * a256x256x64w2x2, a256x128x64w2x2) wherever whole tiles of theirs cover the problem, -1 = never (the ring kernels with
+ * 32x32x16 MFMAs serve every shape, as they do for partly filled tiles). */
+int tl_set_hgemm_agpr_kernels(int mode);
 /* Tuning hook: where the fp32 partial sums of a split-K GEMM are added up.  0 = automatic and 2 = by a second kernel
  * (the default: measured faster on every split shape); 1 = inside the GEMM launch, by the workgroup that finishes a
  * C tile's last split (one counter per tile in the library's scratch, zero between launches), whenever C takes 8-byte

@@ -777,8 +777,9 @@ static const HgemmVariant g_variants[] = {
     TL_HGEMM_PIPE(256, 192, 64, 2, 2, 2),  // 18
     // few rows: four wavefronts of 64x64 read a quarter fewer fragment bytes from LDS than eight of 64x32
     TL_HGEMM_PIPE(128, 128, 64, 2, 2, 4),  // 19
-    // hgemm_big.hip: one wavefront per SIMD, 16x16x32 MFMAs, accumulators in AGPRs (stages < 0 marks it)
+    // hgemm_agpr.hip: one wavefront per SIMD, 16x16x32 MFMAs, accumulators in AGPRs (stages < 0 marks it)
     {"a256x256x64w2x2", 256, 256, 64, 256, -1, nullptr, true, nullptr},  // 20
+    {"a256x128x64w2x2", 256, 128, 64, 256, -2, nullptr, false, nullptr},  // 21
 };
 
 static constexpr int kNumVariants = sizeof(g_variants) / sizeof(g_variants[0]);
@@ -798,6 +799,7 @@ static std::atomic<int> g_forced_band{0};                              // 0 = au
 // stores and come back through device-coherent loads, a serial chain of store acknowledgement, ticket and reload of
 // about 4 us at the end of every tile, where the second kernel reads slabs that still sit in the L2s with every CU.
 static std::atomic<int> g_splitk_merge_mode{0};
+static std::atomic<int> g_agpr_mode{0};   // 0 = the dispatch may take the kernels of hgemm_agpr.hip, -1 = never
 
 // Library-owned fp32 workspace for split-K partial sums, grown on demand (stream-ordered reuse).
 static Workspace g_splitk;
@@ -826,9 +828,11 @@ static bool hgemm_many_rows_split(size_t M, size_t N, size_t K, int cus) {
     return M > 512 && K >= 8192 && t * 2 <= (size_t)cus && t * 22016 <= (size_t)cus * K;
 }
 
-// fast_big: the problem comes in whole 256x256 tiles that hgemm_big.hip's kernel can take (a round of them then costs
+// fast_big: the problem comes in whole 256x256 tiles that hgemm_agpr.hip's kernel can take (a round of them then costs
 // 0.87 of a round of the ring kernel's: 2048x32000x4096 405 against 475 us on one box)
-static HgemmPlan plan_many_rows(size_t M, size_t N, size_t K, int cus, bool can_split, bool fast_big = false) {
+// fast_mid: the same for 128x256 tiles and the 256x128 kernel of that file (0.565 instead of 0.613: 2048x4096x11008 148
+// against 167 us, 2048x2816x4096 50 against 54.5 us, 2048x4096x4096 64.6 against 66.4 us)
+static HgemmPlan plan_many_rows(size_t M, size_t N, size_t K, int cus, bool can_split, bool fast_big = false, bool fast_mid = false) {
     static const int v_big = hgemm_variant_index("p256x256x64w2x4s2");
     static const int v_mid = hgemm_variant_index("p128x256x64w2x4s3");
     static const int v_small = hgemm_variant_index("p128x128x64w2x4s2");
@@ -849,7 +853,7 @@ static HgemmPlan plan_many_rows(size_t M, size_t N, size_t K, int cus, bool can_
         return {v_few_128x128, c_small};
     }
     const double c_big = cost(tiles(256, 256), (size_t)cus, fast_big ? 0.87 : 1.0);
-    const double c_mid = cost(tiles(128, 256), (size_t)cus, 0.613);
+    const double c_mid = cost(tiles(128, 256), (size_t)cus, fast_mid ? 0.565 : 0.613);
     const double c_192 = cost(tiles(256, 192), (size_t)cus, 0.865);   // three quarters of the work at 0.865 of the cost
     int best = v_big;
     double c = c_big;
@@ -899,7 +903,7 @@ static int square_tile_splits(size_t M, size_t N, size_t K, int cus, bool can_sp
     return sp;
 }
 
-static int pick_variant(size_t M, size_t N, size_t K, int cus, bool can_split, bool fast_big = false) {
+static int pick_variant(size_t M, size_t N, size_t K, int cus, bool can_split, bool fast_big = false, bool fast_mid = false) {
     static const int v_big = hgemm_variant_index("p256x256x64w2x4s2");
     static const int v_mid = hgemm_variant_index("p128x256x64w2x4s3");
     static const int v_few_256x128 = hgemm_variant_index("p256x128x64w2x4s3");
@@ -930,7 +934,7 @@ static int pick_variant(size_t M, size_t N, size_t K, int cus, bool can_split, b
         if (tiles(128, 64) > (size_t)cus) return v_few_128x128;
         return v_few_128x64;
     }
-    return plan_many_rows(M, N, K, cus, can_split, fast_big).variant;
+    return plan_many_rows(M, N, K, cus, can_split, fast_big, fast_mid).variant;
 }
 
 // One launch (plus the ordered reduce when K is split) for columns [0, N) of a C whose rows are ldc elements apart.
@@ -958,12 +962,15 @@ int launch_hgemm(const void* A, const void* B, void* C, size_t M, size_t N, size
             if (full >= 1 && rem > 0) {
                 const size_t N1 = full * cols_per_round * 256;
                 const size_t c1 = gate ? N1 / 2 : N1;   // first column of C (and row of B) of the second launch
-                const bool fast_all = gate == 0 && hgemm_big_applies(A, B, C, M, N, K, ldc_all);
-                const bool fast_first = gate == 0 && hgemm_big_applies(A, B, C, M, N1, K, ldc_all);
-                const bool fast_rest = gate == 0 && hgemm_big_applies(A, (const half_t*)B + c1 * K, (half_t*)C + c1, M, N - N1, K, ldc_all);
-                const double whole = plan_many_rows(M, N, K, cus, true, fast_all).cost;
+                const bool agpr_ok = gate == 0 && g_agpr_mode.load() == 0;
+                const bool fast_all = agpr_ok && hgemm_big_applies(A, B, C, M, N, K, ldc_all);
+                const bool fast_first = agpr_ok && hgemm_big_applies(A, B, C, M, N1, K, ldc_all);
+                const bool fast_rest = agpr_ok && hgemm_big_applies(A, (const half_t*)B + c1 * K, (half_t*)C + c1, M, N - N1, K, ldc_all);
+                const bool mid_all = agpr_ok && hgemm_mid_applies(A, B, C, M, N, K, ldc_all);
+                const bool mid_rest = agpr_ok && hgemm_mid_applies(A, (const half_t*)B + c1 * K, (half_t*)C + c1, M, N - N1, K, ldc_all);
+                const double whole = plan_many_rows(M, N, K, cus, true, fast_all, mid_all).cost;
                 const double split = (fast_first ? 0.87 : 1.0) * (double)full * (double)(tiles_m * cols_per_round) / (double)cus +
-                                     plan_many_rows(M, N - N1, K, cus, false, fast_rest).cost + 0.04;   // 0.04: the second launch's ramp
+                                     plan_many_rows(M, N - N1, K, cus, false, fast_rest, mid_rest).cost + 0.04;   // 0.04: the second launch's ramp
                 if (split < whole * 0.97) {
                     int rc = launch_hgemm_cols(A, B, C, M, N1, K, ldc_all, 1, 0, 0, 0, nullptr, nullptr, nullptr, v_big, gate);
                     if (rc != TL_OK) return rc;
@@ -1015,13 +1022,19 @@ static int launch_hgemm_cols(const void* A, const void* B, void* C, size_t M, si
         return launch_hgemm_fewrows(A, B, C, M, N, K, ldc);
     }
     const bool can_split = batch == 1 && ldc == N;   // the second pass of a split K writes a dense C
-    // whole 256x256 tiles of a single dense C: where the 256x256 ring kernel would run, hgemm_big.hip's kernel does
-    const bool fast_big = gate == 0 && batch == 1 && g_forced_variant.load() == 0 && hgemm_big_applies(A, B, C, M, N, K, ldc);
-    int vi = forced_variant ? forced_variant : pick_variant(M, N, K, device_info().cu_count, can_split, fast_big);
+    // whole 256x256 tiles of a single dense C: where the 256x256 ring kernel would run, hgemm_agpr.hip's kernel does
+    const bool agpr_ok = gate == 0 && batch == 1 && g_forced_variant.load() == 0 && g_agpr_mode.load() == 0;
+    const bool fast_big = agpr_ok && hgemm_big_applies(A, B, C, M, N, K, ldc);
+    const bool fast_mid = agpr_ok && M > 512 && hgemm_mid_applies(A, B, C, M, N, K, ldc);
+    int vi = forced_variant ? forced_variant : pick_variant(M, N, K, device_info().cu_count, can_split, fast_big, fast_mid);
     {
         static const int v_big = hgemm_variant_index("p256x256x64w2x4s2");
         static const int v_fast = hgemm_variant_index("a256x256x64w2x2");
+        static const int v_mid = hgemm_variant_index("p128x256x64w2x4s3");
+        static const int v_fast_mid = hgemm_variant_index("a256x128x64w2x2");
         if (fast_big && vi == v_big) vi = v_fast;
+        // (not where the 128x256 ring kernel is about to split K: the 256x128 kernel has no split)
+        if (fast_mid && vi == v_mid && !(can_split && hgemm_many_rows_split(M, N, K, device_info().cu_count))) vi = v_fast_mid;
     }
     int square_splits = 0;
     if (forced_variant == 0 && g_forced_splits.load() == 0) {
@@ -1033,12 +1046,13 @@ static int launch_hgemm_cols(const void* A, const void* B, void* C, size_t M, si
         // whole 256x256 tiles of one dense fp16 C, no gate, no split; anything else falls back to the ring kernel
         const int forced_band = g_forced_band.load();
         const int rt = g_forced_rot_tile.load(), rx = g_forced_rot_xcd.load();
-        if (gate == 0 && batch == 1 && hgemm_big_applies(A, B, C, M, N, K, ldc)) {
+        const bool mid = g_variants[vi].stages == -2;
+        if (gate == 0 && batch == 1 && (mid ? hgemm_mid_applies(A, B, C, M, N, K, ldc) : hgemm_big_applies(A, B, C, M, N, K, ldc))) {
             g_last_variant = vi;
             g_last_splits = 1;
             g_last_one_launch = false;
-            return launch_hgemm_big(A, B, C, M, N, K, ldc, forced_band > 0 ? forced_band : 8, rt >= 0 ? rt : 0,
-                                    rx >= 0 ? rx : (int)(K / 64 / 8));
+            return (mid ? launch_hgemm_mid : launch_hgemm_big)(A, B, C, M, N, K, ldc, forced_band > 0 ? forced_band : 8,
+                                                                rt >= 0 ? rt : 0, rx >= 0 ? rx : (int)(K / 64 / 8));
         }
         static const int v_big = hgemm_variant_index("p256x256x64w2x4s2");
         vi = v_big;
@@ -1256,6 +1270,12 @@ int tl_set_hgemm_k_rotation(int per_tile, int per_xcd) {
 int tl_set_hgemm_tile_band(int band) {
     TL_REQUIRE(band >= 0, "tl_set_hgemm_tile_band: negative band");
     tl::g_forced_band = band;
+    return TL_OK;
+}
+
+int tl_set_hgemm_agpr_kernels(int mode) {
+    TL_REQUIRE(mode == 0 || mode == -1, "tl_set_hgemm_agpr_kernels: %d is not 0 or -1", mode);
+    tl::g_agpr_mode = mode;
     return TL_OK;
 }
 

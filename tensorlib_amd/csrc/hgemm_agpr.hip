@@ -308,6 +308,251 @@ __global__ void __launch_bounds__(256) hgemm_f16_big_kernel(HgemmArgs a) {
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 }
 
+// The same ideas on a 256x128 tile for problems that have too few 256x256 tiles to fill the chip: four wavefronts of
+// 128x64 (128 accumulator registers), a ring of three 48 KB stages (a K tile of this size is multiplied in 1024 cycles,
+// less than a request takes to land, so requests run two tiles ahead), one C tile per workgroup.  Requests for K tiles
+// past the end of K fetch the last K tile again into a stage nobody reads, so every tile of the loop is the same code
+// and the barrier's wait count never changes.  Whole tiles only (M % 256 == 0, N % 128 == 0), K in tiles of 64, at
+// least three.
+#define TL_ACC_FENCE4(acc, i, text) \
+    asm volatile(text : "+a"(acc[i][0]), "+a"(acc[i][1]), "+a"(acc[i][2]), "+a"(acc[i][3]), "+a"(acc[i + 1][0]), \
+                 "+a"(acc[i + 1][1]), "+a"(acc[i + 1][2]), "+a"(acc[i + 1][3]))
+
+template <int A_AHEAD, int BAR_IT, int D_STEP>
+__global__ void __launch_bounds__(256) hgemm_f16_mid_kernel(HgemmArgs a) {
+    constexpr int BM = 256, BN = 128, BK = 64, WN = 2, NW = 4, STAGES = 3;
+    constexpr int RB = BK * 2;
+    constexpr int CPR = BK / 8;
+    constexpr int RPL = 256 / RB;
+    constexpr int RPW = 1024 / RB;
+    constexpr int A_REQS = BM / RPW / NW;      // 8
+    constexpr int B_REQS = BN / RPW / NW;      // 4
+    constexpr int NREQ = A_REQS + B_REQS;
+    constexpr int A_BYTES = BM * RB;
+    constexpr int STAGE_BYTES = (BM + BN) * RB;
+    constexpr int TM = 128, TN = 64;           // wavefront tile
+    constexpr int MT = TM / 16, NT = TN / 16;
+    constexpr int KS = BK / 32;
+    constexpr int SLOTS = KS * MT * NT;        // 64 MFMAs per K tile
+    constexpr int NA = KS * MT;
+    static_assert((NW * RPW / RPL) % CPR == 0, "the chunk a lane fetches must not depend on the request");
+    constexpr int BARRIER_SLOT = BAR_IT * NT;
+    static_assert(A_AHEAD >= 1 && NA - 1 - A_AHEAD < BAR_IT && BAR_IT < NA, "the last A fragment is requested before the barrier");
+    static_assert(BARRIER_SLOT + 1 + NT + A_AHEAD <= SLOTS, "the next tile's first fragments are read behind the barrier");
+    // request d < EARLY of K tile kt+3 goes out behind MFMA BARRIER_SLOT + 1 + D_STEP d of tile kt (the barrier has just
+    // freed its stage), the others behind MFMA 1 + D_STEP (d - EARLY) of tile kt+1; at the barrier of tile kt+1 all of
+    // them are out and may be in flight, everything older has to have landed
+    constexpr int EARLY_ROOM = (SLOTS - BARRIER_SLOT - 2) / D_STEP + 1;
+    constexpr int EARLY = EARLY_ROOM < NREQ ? EARLY_ROOM : NREQ;
+    constexpr int LATE = NREQ - EARLY;
+    static_assert(LATE == 0 || 1 + D_STEP * (LATE - 1) < BARRIER_SLOT, "a tile's requests are out before the next barrier");
+
+    extern __shared__ __attribute__((aligned(1024))) unsigned char smem_raw[];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave / WN, wn = wave % WN;
+    const int K = a.K, ldc = a.ldc;
+    half_t* __restrict__ C = a.C;
+    const int KT = K / BK;
+    const size_t row_bytes = (size_t)K * 2;
+
+    int tm, tn;
+    tile_of_block(blockIdx.x, a.tiles_m * a.tiles_n, a.tiles_m, a.band_m, tm, tn);
+    const unsigned char* const a_tile = reinterpret_cast<const unsigned char*>(a.A) + (size_t)tm * BM * row_bytes;
+    const unsigned char* const b_tile = reinterpret_cast<const unsigned char*>(a.B) + (size_t)tn * BN * row_bytes;
+    const int rot = (int)(((unsigned)tn * (unsigned)a.rot_tile + (blockIdx.x & 7u) * (unsigned)a.rot_xcd) % (unsigned)KT);
+
+    const int r0 = wave * RPW + lane / CPR;
+    const int chunk = (lane % CPR) ^ ((r0 / RPL) % CPR);
+    unsigned req_off[A_REQS];
+#pragma unroll
+    for (int d = 0; d < A_REQS; ++d) req_off[d] = (unsigned)(((size_t)(r0 + d * NW * RPW) * K + (size_t)chunk * 8) * 2);
+    const unsigned lds_wave = (unsigned)(unsigned long)(__attribute__((address_space(3))) unsigned char*)smem_raw + (unsigned)wave * 1024u;
+
+    // the request stream: K tile `req_pos` of the walk (clamped to the last one), as base pointers into A and B
+    int req_pos = 0, req_k = rot;
+    const unsigned char *req_a = a_tile + (size_t)req_k * (BK * 2), *req_b = b_tile + (size_t)req_k * (BK * 2);
+    const unsigned char *late_a = req_a, *late_b = req_b;
+    auto req_advance = [&]() {
+        late_a = req_a;
+        late_b = req_b;
+        ++req_pos;
+        if (req_pos < KT) {
+            ++req_k;
+            if (req_k == KT) req_k = 0;
+            req_a = a_tile + (size_t)req_k * (BK * 2);
+            req_b = b_tile + (size_t)req_k * (BK * 2);
+        }
+    };
+    auto request = [&](auto dd, auto stage, const unsigned char* pa, const unsigned char* pb) {
+        constexpr int d = decltype(dd)::value, st = decltype(stage)::value;
+        if constexpr (d < A_REQS)
+            request_16B_per_lane<st * STAGE_BYTES + d * NW * 1024>(pa, req_off[d], lds_wave);
+        else
+            request_16B_per_lane<st * STAGE_BYTES + A_BYTES + (d - A_REQS) * NW * 1024>(pb, req_off[d - A_REQS], lds_wave);
+    };
+
+    const int fr_row = lane & 15;
+    const int fr_sw = (fr_row / RPL) % CPR;
+    int fr_off[KS];
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) fr_off[ks] = fr_row * RB + (((ks * 4 + (lane >> 4)) ^ fr_sw) * 16);
+    const unsigned char* const a_frag = smem_raw + wm * TM * RB;
+    const unsigned char* const b_frag = smem_raw + A_BYTES + wn * TN * RB;
+
+    float4_t acc[MT][NT];
+    half8_t abuf[NA];
+    half8_t bbuf[2][NT];
+    using S0 = std::integral_constant<int, 0>;
+    using S1 = std::integral_constant<int, 1>;
+    using S2 = std::integral_constant<int, 2>;
+
+    // prologue: K tiles 0 and 1 whole, the early requests of K tile 2; tile 0 has to have landed
+    static_for<0, NREQ>([&](auto d) { request(d, S0{}, req_a, req_b); });
+    req_advance();
+    static_for<0, NREQ>([&](auto d) { request(d, S1{}, req_a, req_b); });
+    req_advance();
+    static_for<0, EARLY>([&](auto d) { request(d, S2{}, req_a, req_b); });
+    req_advance();
+    asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(NREQ + EARLY) : "memory");
+    abuf[0] = *reinterpret_cast<const half8_t*>(a_frag + fr_off[0]);
+#pragma unroll
+    for (int j = 0; j < NT; ++j) bbuf[0][j] = *reinterpret_cast<const half8_t*>(b_frag + j * 16 * RB + fr_off[0]);
+#pragma unroll
+    for (int n = 1; n < A_AHEAD; ++n) abuf[n] = *reinterpret_cast<const half8_t*>(a_frag + n * 16 * RB + fr_off[0]);
+
+    // One K tile in stage P; the next one is in stage (P + 1) % 3, the requests of the tile after that are finishing in
+    // stage (P + 2) % 3, and behind the barrier stage P takes the first requests of the tile three ahead.
+    auto tile = [&](auto par, auto first) {
+        constexpr int P = decltype(par)::value;
+        constexpr bool FIRST = decltype(first)::value;
+        using Cur = std::integral_constant<int, P>;
+        using Aft = std::integral_constant<int, (P + 2) % STAGES>;
+        const unsigned char* const a_cur = a_frag + P * STAGE_BYTES;
+        const unsigned char* const b_cur = b_frag + P * STAGE_BYTES;
+        const unsigned char* const a_nxt = a_frag + ((P + 1) % STAGES) * STAGE_BYTES;
+        const unsigned char* const b_nxt = b_frag + ((P + 1) % STAGES) * STAGE_BYTES;
+        static_for<0, SLOTS>([&](auto slot) {
+            constexpr int q = decltype(slot)::value;
+            constexpr int s = q / (MT * NT), i = (q / NT) % MT, j = q % NT, n = s * MT + i;
+            // tile kt+1 has landed for this wavefront (the NREQ requests of tile kt+2 may be in flight), its LDS reads
+            // of tile kt are done; behind the barrier that holds for everyone
+            if constexpr (q == BARRIER_SLOT) asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(NREQ) : "memory");
+            if constexpr (FIRST && s == 0) mfma_agpr_first(acc[i][j], bbuf[s][j], abuf[n]);
+            else mfma_agpr(acc[i][j], bbuf[s][j], abuf[n]);
+            if constexpr (j == 0 && n + A_AHEAD < NA) {
+                constexpr int n2 = n + A_AHEAD;
+                abuf[n2] = *reinterpret_cast<const half8_t*>(a_cur + (n2 % MT) * 16 * RB + fr_off[n2 / MT]);
+            }
+            if constexpr (s + 1 < KS && j == 2 && i < NT)
+                bbuf[(s + 1) % KS][i] = *reinterpret_cast<const half8_t*>(b_cur + i * 16 * RB + fr_off[(s + 1) % KS]);
+            // r-th read behind the barrier: A0, B0 .. B(NT-1), A1 ..
+            if constexpr (q > BARRIER_SLOT && q - BARRIER_SLOT - 1 < NT + A_AHEAD) {
+                constexpr int r = q - BARRIER_SLOT - 1;
+                if constexpr (r == 0) abuf[0] = *reinterpret_cast<const half8_t*>(a_nxt + fr_off[0]);
+                else if constexpr (r <= NT) bbuf[0][r - 1] = *reinterpret_cast<const half8_t*>(b_nxt + (r - 1) * 16 * RB + fr_off[0]);
+                else abuf[r - NT] = *reinterpret_cast<const half8_t*>(a_nxt + (r - NT) * 16 * RB + fr_off[0]);
+            }
+            if constexpr (q >= 1 && (q - 1) % D_STEP == 0 && (q - 1) / D_STEP < LATE)
+                request(std::integral_constant<int, EARLY + (q - 1) / D_STEP>{}, Aft{}, late_a, late_b);
+            if constexpr (q > BARRIER_SLOT && (q - BARRIER_SLOT - 1) % D_STEP == 0 && (q - BARRIER_SLOT - 1) / D_STEP < EARLY)
+                request(std::integral_constant<int, (q - BARRIER_SLOT - 1) / D_STEP>{}, Cur{}, req_a, req_b);
+            __builtin_amdgcn_sched_barrier(0);
+        });
+        req_advance();
+    };
+
+    {
+        using T = std::true_type;
+        using F = std::false_type;
+        tile(S0{}, T{});
+        int kt = 1;
+        for (; kt + 3 <= KT; kt += 3) {
+            tile(S1{}, F{});
+            tile(S2{}, F{});
+            tile(S0{}, F{});
+        }
+        if (kt < KT) {
+            tile(S1{}, F{});
+            if (kt + 1 < KT) tile(S2{}, F{});
+        }
+    }
+    TL_ACC_FENCE4(acc, 0, "s_nop 15\n\ts_nop 15");
+    TL_ACC_FENCE4(acc, 2, "");
+    TL_ACC_FENCE4(acc, 4, "");
+    TL_ACC_FENCE4(acc, 6, "");
+
+    // ---- epilogue, as in the 256x256 kernel: 16 x TN blocks through a private LDS region behind the ring ----
+    const int e_row = lane & 15;
+    const int e_col = (lane >> 4) * 4;
+    const int row_base = tm * BM + wm * TM, col_base = tn * BN + wn * TN;
+    constexpr int RS = TN * 2 + 16;
+    constexpr int CH = TN / 8;
+    constexpr int RPR = 64 / CH;
+    constexpr int PASSES = 16 / RPR;
+    static_assert(64 % CH == 0 && 16 % RPR == 0, "a staged block is read back in whole wavefront-wide passes");
+    unsigned char* region = smem_raw + STAGES * STAGE_BYTES + wave * (16 * RS);
+#pragma unroll
+    for (int i = 0; i < MT; ++i) {
+#pragma unroll
+        for (int j = 0; j < NT; ++j) {
+            half4_t h = {(half_t)acc[i][j][0], (half_t)acc[i][j][1], (half_t)acc[i][j][2], (half_t)acc[i][j][3]};
+            *reinterpret_cast<half4_t*>(region + e_row * RS + (j * 16 + e_col) * 2) = h;
+        }
+#pragma unroll
+        for (int q = 0; q < PASSES; ++q) {
+            const int r = q * RPR + lane / CH, c = lane % CH;
+            const half8_t v = *reinterpret_cast<const half8_t*>(region + r * RS + c * 16);
+            const int row = row_base + i * 16 + r, col = col_base + c * 8;
+            *reinterpret_cast<half8_t*>(C + (size_t)row * ldc + col) = v;
+        }
+    }
+    // the requests past the end of K may still be in flight towards LDS
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+}
+
+static std::atomic<bool> g_mid_attr{false};
+
+const char* hgemm_mid_name() { return "a256x128x64w2x2"; }
+
+bool hgemm_mid_applies(const void* A, const void* B, const void* C, size_t M, size_t N, size_t K, size_t ldc) {
+    return M >= 256 && N >= 128 && M % 256 == 0 && N % 128 == 0 && K >= 192 && K % 64 == 0 && K <= ((size_t)1 << 22) &&
+           ldc % 8 == 0 && ldc >= N && aligned16(A) && aligned16(B) && aligned16(C) && M <= 0x7fffffffu && N <= 0x7fffffffu;
+}
+
+int launch_hgemm_mid(const void* A, const void* B, void* C, size_t M, size_t N, size_t K, size_t ldc, int band, int rot_tile,
+                     int rot_xcd) {
+    TL_REQUIRE(hgemm_mid_applies(A, B, C, M, N, K, ldc), "hgemm: %s does not serve this shape", hgemm_mid_name());
+    void (*const kernel)(HgemmArgs) = hgemm_f16_mid_kernel<3, 13, 4>;
+    // the three-stage ring and behind it the C staging of the epilogue (four wavefronts x 16 rows x (128 + 16) bytes)
+    const size_t lds = (size_t)3 * (256 + 128) * 64 * sizeof(half_t) + (size_t)4 * 16 * (64 * 2 + 16);
+    if (!g_mid_attr.load()) {
+        TL_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+        g_mid_attr.store(true);
+    }
+    HgemmArgs a{};
+    a.A = (const half_t*)A;
+    a.B = (const half_t*)B;
+    a.C = (half_t*)C;
+    a.M = (int)M;
+    a.N = (int)N;
+    a.K = (int)K;
+    a.ldc = (int)ldc;
+    a.tiles_m = (int)(M / 256);
+    a.tiles_n = (int)(N / 128);
+    a.kt_per_split = 0x7fffffff;
+    a.band_m = band > 0 ? band : 8;
+    a.rot_tile = rot_tile;
+    a.rot_xcd = rot_xcd;
+    const size_t nblocks = (size_t)a.tiles_m * a.tiles_n;
+    TL_REQUIRE(nblocks <= 0x7fffffffu, "hgemm: too many tiles");
+    hipLaunchKernelGGL(kernel, dim3((unsigned)nblocks), dim3(256), lds, stream(), a);
+    TL_CHECK_LAUNCH(hgemm_mid_name());
+    return TL_OK;
+}
+
 static std::atomic<bool> g_big_attr{false};
 
 const char* hgemm_big_name() { return "a256x256x64w2x2"; }

@@ -767,10 +767,10 @@ def test_hgemm_split_k_falls_back_to_the_second_kernel(dev):
 BASELINE_PLANS = [
     # (M, N, K), (variant of the last launch, K splits): the twelve prefill shapes and the four projections of a 16-token
     # prompt on a 256-CU MI355X
-    ((2048, 4096, 4096), ("p128x256x64w2x4s3", 1)),
-    ((2048, 11008, 4096), ("p128x256x64w2x4s3", 1)),   # 8192 columns of 256x256 tiles first, this is the launch for the rest
+    ((2048, 4096, 4096), ("a256x128x64w2x2", 1)),
+    ((2048, 11008, 4096), ("a256x128x64w2x2", 1)),   # 8192 columns of 256x256 tiles first, this is the launch for the rest
     ((2048, 32000, 4096), ("a256x256x64w2x2", 1)),
-    ((2048, 4096, 11008), ("p128x256x64w2x4s3", 1)),
+    ((2048, 4096, 11008), ("a256x128x64w2x2", 1)),
     ((512, 4096, 4096), ("p128x64x64w4x1s4", 1)),
     ((512, 11008, 4096), ("p128x192x64w4x2s4", 1)),
     ((512, 32000, 4096), ("a256x256x64w2x2", 1)),
@@ -827,17 +827,57 @@ def test_hgemm_256x256_agpr_kernel_integer_exact(dev, shape):
         dev.lib.tl_set_hgemm_k_rotation(-1, -1)
 
 
+@pytest.mark.parametrize("shape", [(256, 128, 192), (256, 128, 256), (512, 384, 320), (2048, 4096, 448), (2560, 11008, 1024),
+                                   (256, 256, 11008)], ids=lambda s: "x".join(map(str, s)))
+def test_hgemm_256x128_agpr_kernel_integer_exact(dev, shape):
+    """hgemm_f16_mid_kernel forced on whole-tile shapes with 3, 4, 5, 7, 16 and 172 K tiles (every remainder of the
+    three-stage ring's unrolled loop), one tile, more tiles than compute units, rotated K walks: small integers are
+    exact whatever the order, so a K tile skipped, repeated or read from the wrong stage shows as a wrong bit."""
+    M, N, K = shape
+    A = dev.from_numpy(synth.small_ints_f16(9400 + M, (M, K), -2, 2))
+    B = dev.from_numpy(synth.small_ints_f16(9401 + N % 83, (N, K), -2, 2))
+    want = A.double() @ B.double().T
+    assert float(want.abs().max()) <= 2048
+    V = dev.hgemm_variants().index("a256x128x64w2x2")
+    try:
+        dev.set_hgemm_variant(V)
+        for rot in ((-1, -1), (0, 0), (3, 5), (1000003, 17)):
+            dev.lib.tl_set_hgemm_k_rotation(*rot)
+            C = dev.hgemm(A, B)
+            assert dev.hgemm_last_plan() == ("a256x128x64w2x2", 1)
+            assert torch.equal(C.double(), want), (shape, rot)
+    finally:
+        dev.set_hgemm_variant(0)
+        dev.lib.tl_set_hgemm_k_rotation(-1, -1)
+
+
+def test_hgemm_agpr_kernels_can_be_switched_off(dev):
+    """tl_set_hgemm_agpr_kernels(-1) hands the shapes back to the ring kernels; both give the exact integer result."""
+    A = dev.from_numpy(synth.small_ints_f16(9500, (2048, 512), -2, 2))
+    B = dev.from_numpy(synth.small_ints_f16(9501, (8192, 512), -2, 2))
+    want = A.double() @ B.double().T
+    try:
+        C = dev.hgemm(A, B)
+        assert dev.hgemm_last_plan()[0].startswith("a256x") and torch.equal(C.double(), want)
+        dev.lib.tl_set_hgemm_agpr_kernels(-1)
+        C = dev.hgemm(A, B)
+        assert dev.hgemm_last_plan()[0].startswith("p") and torch.equal(C.double(), want)
+    finally:
+        dev.lib.tl_set_hgemm_agpr_kernels(0)
+
+
 def test_hgemm_256x256_agpr_kernel_falls_back_on_partial_tiles(dev, oracle):
     """Rows or columns that do not fill whole 256x256 tiles, a K that is not an even number of tiles: the forced variant
     hands the call to the ring kernel."""
-    V = dev.hgemm_variants().index("a256x256x64w2x2")
+    names = dev.hgemm_variants()
     try:
-        dev.set_hgemm_variant(V)
-        for (M, N, K) in [(300, 512, 256), (512, 520, 256), (512, 512, 192), (256, 256, 128)]:
-            A = synth.small_ints_f16(9300 + M, (M, K), -2, 2)
-            B = synth.small_ints_f16(9301 + N, (N, K), -2, 2)
-            C = dev.hgemm(dev.from_numpy(A), dev.from_numpy(B)).cpu().numpy()
-            assert dev.hgemm_last_plan()[0] != "a256x256x64w2x2"
-            assert np.array_equal(C.view(np.uint16), oracle.matmul2d(A, B).view(np.uint16)), (M, N, K)
+        for name in ("a256x256x64w2x2", "a256x128x64w2x2"):
+            dev.set_hgemm_variant(names.index(name))
+            for (M, N, K) in [(300, 512, 256), (512, 520, 256), (512, 512, 160), (256, 256, 128)]:
+                A = synth.small_ints_f16(9300 + M, (M, K), -2, 2)
+                B = synth.small_ints_f16(9301 + N, (N, K), -2, 2)
+                C = dev.hgemm(dev.from_numpy(A), dev.from_numpy(B)).cpu().numpy()
+                assert dev.hgemm_last_plan()[0] != name
+                assert np.array_equal(C.view(np.uint16), oracle.matmul2d(A, B).view(np.uint16)), (name, M, N, K)
     finally:
         dev.set_hgemm_variant(0)
