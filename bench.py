@@ -183,10 +183,12 @@ def time_region(fn, reps: int, torch):
 
 
 def mfma_sustained(dev):
-    """MFMA rate out of registers: constant operands vs operands changing with every instruction."""
+    """MFMA rate out of registers: constant operands vs operands changing with every instruction, for the 32x32x16
+    instruction (the ring kernels') and the 16x16x32 one (the AGPR kernels')."""
     import ctypes
     out = {}
-    for name, mode in (("constant_operands", 0), ("changing_operands", 1)):
+    for name, mode in (("constant_operands", 0), ("changing_operands", 1), ("constant_operands_16x16x32", 2),
+                       ("changing_operands_16x16x32", 3)):
         v = ctypes.c_double()
         from tensorlib_amd._lib import check
         check(dev.lib.tl_measure_mfma_rate_f16(mode, ctypes.byref(v)), "tl_measure_mfma_rate_f16")
@@ -217,7 +219,8 @@ def hgemm_table(dev, randn, torch, synth, sustained_tf, shapes=None):
         tf = synth.gemm_flops(M, N, K) / us / 1e6
         ai = synth.gemm_flops(M, N, K) / synth.gemm_min_bytes(M, N, K)
         bound_tf = min(MFMA_FP16_PEAK_TFLOPS, ai * HBM_PEAK_GBS / 1e3)
-        hg[f"{M}x{N}x{K}"] = {"us": round(us, 1), "TFLOP/s": round(tf, 1),
+        plan = dev.hgemm_last_plan()
+        hg[f"{M}x{N}x{K}"] = {"us": round(us, 1), "TFLOP/s": round(tf, 1), "kernel": plan[0], "k_splits": plan[1],
                               "frac_mfma_peak": round(tf / MFMA_FP16_PEAK_TFLOPS, 4),
                               "bound": "mfma" if bound_tf >= MFMA_FP16_PEAK_TFLOPS else "hbm",
                               "frac_of_bound": round(tf / bound_tf, 4),
@@ -403,12 +406,14 @@ def main():
                        "splitk_merge": args.splitk_merge, "variant": args.hgemm_variant or "dispatch"},
             "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": MFMA_FP16_PEAK_TFLOPS, "unit": "TFLOP/s",
                          "frac": round(achieved / MFMA_FP16_PEAK_TFLOPS, 4), "traffic": None,
-                         "kernel": "hgemm_f16_dlds_kernel", "flops_per_launch": step_flops / len(shapes),
+                         "kernel": "by shape: hgemm_f16_big_kernel / hgemm_f16_mid_kernel (a256x..), hgemm_f16_dlds_kernel (p..), "
+                                   "hgemm_fewrows_kernel (fewrows); extra.hgemm_prefill names it per shape",
+                         "flops_per_launch": step_flops / len(shapes),
                          "avg_launch_us": round(ev / args.steps / len(shapes) * 1e6, 2),
                          "sustained_mfma_tflops": sustained},
         }
         if not args.no_extra:
-            out["extra"] = {"hgemm_prefill": hgemm_table(dev, randn, torch, synth, sustained["changing_operands"], shapes)}
+            out["extra"] = {"hgemm_prefill": hgemm_table(dev, randn, torch, synth, max(sustained["changing_operands"], sustained["changing_operands_16x16x32"]), shapes)}
         if not args.no_cpu:
             out["cpu_baseline"] = cpu_baseline_hgemm()
         print(json.dumps(out))
@@ -522,9 +527,9 @@ def main():
 
         sustained = mfma_sustained(dev)
         extra["mfma_sustained_tflops"] = sustained
-        extra["hgemm_prefill"] = hgemm_table(dev, randn, torch, synth, sustained["changing_operands"])
+        extra["hgemm_prefill"] = hgemm_table(dev, randn, torch, synth, max(sustained["changing_operands"], sustained["changing_operands_16x16x32"]))
         # a prompt of a few tokens (the reference's usual prefill): the projections of a 16-token prompt
-        extra["hgemm_short_prompt"] = hgemm_table(dev, randn, torch, synth, sustained["changing_operands"],
+        extra["hgemm_short_prompt"] = hgemm_table(dev, randn, torch, synth, max(sustained["changing_operands"], sustained["changing_operands_16x16x32"]),
                                                   [(16, 12288, 4096), (16, 4096, 4096), (16, 22016, 4096), (16, 4096, 11008)])
         torch.cuda.empty_cache()
         from tensorlib_amd import llama2

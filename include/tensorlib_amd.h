@@ -353,8 +353,11 @@ int tl_silu_mul_rows_f16(void* out, const void* ab, size_t rows, size_t hidden);
 
 /* out[M, hidden] = silu(X . W1^T) * (X . W3^T) for W13 = [W1; W3] stored as one [2*hidden, K] matrix: the two
  * projections and the gate of FeedForward::forward (model/llama2_7b/src/Transformer.cpp:136-141) in one launch, the
- * gate applied to the fp16-rounded projections in the GEMM's epilogue (same bits as tl_matmul2d_f16 into a
- * [M, 2*hidden] buffer followed by tl_silu_mul_rows_f16).  Shapes the one-launch kernel does not serve (K % 64 != 0,
+ * gate applied to the fp16-rounded projections in the GEMM's epilogue: the arithmetic of tl_matmul2d_f16 into a
+ * [M, 2*hidden] buffer followed by tl_silu_mul_rows_f16.  The bits agree with that pair when both add the products
+ * of a row in the same order (the same kernel family, K walked from the same first tile, K not split: what
+ * tl_set_hgemm_k_rotation(0, 0) and tl_set_hgemm_splits(1) force); the default dispatch picks tiles and K walks per
+ * launch, so the two generally differ by the rounding of the fp32 sums, within the tolerance of the GEMM.  Shapes the one-launch kernel does not serve (K % 64 != 0,
  * unaligned pointers, at most 32 rows, M == 1) take exactly that two-step path through `scratch`
  * ([M, 2*hidden] halves; may be NULL when the caller knows the one-launch path applies).  hidden % 8 == 0. */
 int tl_hgemm_silu_mul_f16(const void* X, const void* W13, void* scratch, void* out, size_t M, size_t hidden, size_t K);

@@ -1182,9 +1182,15 @@ int tl_hgemm_prefill_rope_qkv_vt_f16(const void* X, const void* Wqkv, void* qkv,
                                      const void* rope_table, void* vT, int ldv, int n_tokens, int n_heads, int head_dim,
                                      size_t K) {
     TL_ENSURE_INIT();
-    TL_REQUIRE(X && Wqkv && qkv, "tl_hgemm_prefill_rope_qkv_vt_f16: null pointer");
+    // every argument of both steps is checked before the first launch: a rejected call has written nothing
+    TL_REQUIRE(X && Wqkv && qkv && q_out && cache_k && cache_v && rope_table && vT, "tl_hgemm_prefill_rope_qkv_vt_f16: null pointer");
     TL_REQUIRE(n_tokens >= 1 && n_heads >= 1 && (head_dim == 64 || head_dim == 128),
                "tl_hgemm_prefill_rope_qkv_vt_f16: bad sizes");
+    TL_REQUIRE(n_heads <= 65535 && ldv % 64 == 0 && ldv >= n_tokens,
+               "tl_hgemm_prefill_rope_qkv_vt_f16: ldv=%d must be a multiple of 64 that covers the tokens", ldv);
+    TL_REQUIRE(tl::aligned16(q_out) && tl::aligned16(qkv) && tl::aligned16(cache_k) && tl::aligned16(cache_v) &&
+                   tl::aligned16(rope_table) && tl::aligned16(vT),
+               "tl_hgemm_prefill_rope_qkv_vt_f16: pointers must be 16-byte aligned");
     const size_t dim = (size_t)n_heads * head_dim, N = 3 * dim, M = (size_t)n_tokens;
     float* slabs = nullptr;
     int splits = 1;
@@ -1196,13 +1202,8 @@ int tl_hgemm_prefill_rope_qkv_vt_f16(const void* X, const void* Wqkv, void* qkv,
     if (splits <= 1)
         return tl_prefill_rope_qkv_vt_f16(q_out, base, base + dim, base + 2 * dim, N, cache_k, cache_v, rope_table, vT, ldv,
                                           n_tokens, n_heads, head_dim);
-    // same argument checks as the entry above, the projections read from the slabs
-    TL_REQUIRE(q_out && cache_k && cache_v && rope_table && vT, "tl_hgemm_prefill_rope_qkv_vt_f16: null pointer");
-    TL_REQUIRE(n_heads <= 65535 && ldv % 64 == 0 && ldv >= n_tokens,
-               "tl_hgemm_prefill_rope_qkv_vt_f16: ldv=%d must be a multiple of 64 that covers the tokens", ldv);
-    TL_REQUIRE(tl::aligned16(q_out) && tl::aligned16(cache_k) && tl::aligned16(cache_v) && tl::aligned16(rope_table) &&
-                   tl::aligned16(vT) && tl::aligned16(slabs),
-               "tl_hgemm_prefill_rope_qkv_vt_f16: pointers must be 16-byte aligned");
+    // the projections read from the slabs
+    TL_REQUIRE(tl::aligned16(slabs), "tl_hgemm_prefill_rope_qkv_vt_f16: the split-K slabs must be 16-byte aligned");
     dim3 grid((unsigned)(ldv / 64), (unsigned)n_heads, 3);
     auto column = [](size_t col) { return reinterpret_cast<const tl::half_t*>((uintptr_t)(col * sizeof(tl::half_t))); };
     auto launch = [&](auto kernel) {

@@ -962,12 +962,12 @@ int launch_hgemm(const void* A, const void* B, void* C, size_t M, size_t N, size
             if (full >= 1 && rem > 0) {
                 const size_t N1 = full * cols_per_round * 256;
                 const size_t c1 = gate ? N1 / 2 : N1;   // first column of C (and row of B) of the second launch
-                const bool agpr_ok = gate == 0 && g_agpr_mode.load() == 0;
-                const bool fast_all = agpr_ok && hgemm_big_applies(A, B, C, M, N, K, ldc_all);
-                const bool fast_first = agpr_ok && hgemm_big_applies(A, B, C, M, N1, K, ldc_all);
-                const bool fast_rest = agpr_ok && hgemm_big_applies(A, (const half_t*)B + c1 * K, (half_t*)C + c1, M, N - N1, K, ldc_all);
-                const bool mid_all = agpr_ok && hgemm_mid_applies(A, B, C, M, N, K, ldc_all);
-                const bool mid_rest = agpr_ok && hgemm_mid_applies(A, (const half_t*)B + c1 * K, (half_t*)C + c1, M, N - N1, K, ldc_all);
+                const bool agpr_ok = g_agpr_mode.load() == 0;   // (the 256x128 kernel has no gated build)
+                const bool fast_all = agpr_ok && hgemm_big_applies(A, B, C, M, N, K, ldc_all, gate);
+                const bool fast_first = agpr_ok && hgemm_big_applies(A, B, C, M, N1, K, ldc_all, gate);
+                const bool fast_rest = agpr_ok && hgemm_big_applies(A, (const half_t*)B + c1 * K, (half_t*)C + c1, M, N - N1, K, ldc_all, gate);
+                const bool mid_all = agpr_ok && gate == 0 && hgemm_mid_applies(A, B, C, M, N, K, ldc_all);
+                const bool mid_rest = agpr_ok && gate == 0 && hgemm_mid_applies(A, (const half_t*)B + c1 * K, (half_t*)C + c1, M, N - N1, K, ldc_all);
                 const double whole = plan_many_rows(M, N, K, cus, true, fast_all, mid_all).cost;
                 const double split = (fast_first ? 0.87 : 1.0) * (double)full * (double)(tiles_m * cols_per_round) / (double)cus +
                                      plan_many_rows(M, N - N1, K, cus, false, fast_rest, mid_rest).cost + 0.04;   // 0.04: the second launch's ramp
@@ -1023,9 +1023,9 @@ static int launch_hgemm_cols(const void* A, const void* B, void* C, size_t M, si
     }
     const bool can_split = batch == 1 && ldc == N;   // the second pass of a split K writes a dense C
     // whole 256x256 tiles of a single dense C: where the 256x256 ring kernel would run, hgemm_agpr.hip's kernel does
-    const bool agpr_ok = gate == 0 && batch == 1 && g_forced_variant.load() == 0 && g_agpr_mode.load() == 0;
-    const bool fast_big = agpr_ok && hgemm_big_applies(A, B, C, M, N, K, ldc);
-    const bool fast_mid = agpr_ok && M > 512 && hgemm_mid_applies(A, B, C, M, N, K, ldc);
+    const bool agpr_ok = batch == 1 && g_forced_variant.load() == 0 && g_agpr_mode.load() == 0;
+    const bool fast_big = agpr_ok && hgemm_big_applies(A, B, C, M, N, K, ldc, gate);
+    const bool fast_mid = agpr_ok && gate == 0 && M > 512 && hgemm_mid_applies(A, B, C, M, N, K, ldc);
     int vi = forced_variant ? forced_variant : pick_variant(M, N, K, device_info().cu_count, can_split, fast_big, fast_mid);
     {
         static const int v_big = hgemm_variant_index("p256x256x64w2x4s2");
@@ -1043,16 +1043,17 @@ static int launch_hgemm_cols(const void* A, const void* B, void* C, size_t M, si
         if (square_splits > 0) vi = v_square;
     }
     if (g_variants[vi].stages < 0) {
-        // whole 256x256 tiles of one dense fp16 C, no gate, no split; anything else falls back to the ring kernel
+        // whole tiles of one fp16 C, no split (and no gate on the 256x128 tile); anything else falls back to the ring kernel
         const int forced_band = g_forced_band.load();
         const int rt = g_forced_rot_tile.load(), rx = g_forced_rot_xcd.load();
         const bool mid = g_variants[vi].stages == -2;
-        if (gate == 0 && batch == 1 && (mid ? hgemm_mid_applies(A, B, C, M, N, K, ldc) : hgemm_big_applies(A, B, C, M, N, K, ldc))) {
+        const int band = forced_band > 0 ? forced_band : 8, rot_tile = rt >= 0 ? rt : 0, rot_xcd = rx >= 0 ? rx : (int)(K / 64 / 8);
+        if (batch == 1 && (mid ? gate == 0 && hgemm_mid_applies(A, B, C, M, N, K, ldc) : hgemm_big_applies(A, B, C, M, N, K, ldc, gate))) {
             g_last_variant = vi;
             g_last_splits = 1;
             g_last_one_launch = false;
-            return (mid ? launch_hgemm_mid : launch_hgemm_big)(A, B, C, M, N, K, ldc, forced_band > 0 ? forced_band : 8,
-                                                                rt >= 0 ? rt : 0, rx >= 0 ? rx : (int)(K / 64 / 8));
+            return mid ? launch_hgemm_mid(A, B, C, M, N, K, ldc, band, rot_tile, rot_xcd)
+                       : launch_hgemm_big(A, B, C, M, N, K, ldc, band, rot_tile, rot_xcd, gate);
         }
         static const int v_big = hgemm_variant_index("p256x256x64w2x4s2");
         vi = v_big;

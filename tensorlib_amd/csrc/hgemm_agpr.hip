@@ -84,7 +84,10 @@ __device__ __forceinline__ void request_16B_per_lane(const void* uniform_base, u
 
 // A_AHEAD: how many iterations (of NT MFMAs) ahead of its use an A fragment is read; BAR_IT: the iteration in front of
 // which the K tile's barrier stands; D_STEP: MFMAs between two requests.
-template <int A_AHEAD, int BAR_IT, int D_STEP>
+// GATED: the SwiGLU gate in the epilogue, as in the gated build of hgemm_f16_dlds_kernel (HgemmArgs::gate).  A B tile
+// then holds, per wavefront column, 64 rows of the first matrix followed by the 64 rows of the second one that pair
+// with them, and covers 128 columns of C; the host passes tiles_n and ldc in output columns.
+template <int A_AHEAD, int BAR_IT, int D_STEP, bool GATED>
 __global__ void __launch_bounds__(256) hgemm_f16_big_kernel(HgemmArgs a) {
     constexpr int BM = 256, BN = 256, BK = 64, WN = 2, NW = 4;
     constexpr int RB = BK * 2;                 // bytes per tile row
@@ -142,6 +145,18 @@ __global__ void __launch_bounds__(256) hgemm_f16_big_kernel(HgemmArgs a) {
     unsigned req_off[A_REQS];
 #pragma unroll
     for (int d = 0; d < A_REQS; ++d) req_off[d] = (unsigned)(((size_t)(r0 + d * NW * RPW) * K + (size_t)chunk * 8) * 2);
+    // gated: tile row r of B is row (r / TN) * (TN / 2) + r % (TN / 2) of the tile's 128 output columns, taken from the
+    // first matrix for the first half of a wavefront column and `gate` rows further down for the second half
+    unsigned req_off_gated[GATED ? B_REQS : 1];
+    if constexpr (GATED) {
+#pragma unroll
+        for (int d = 0; d < B_REQS; ++d) {
+            const int r = r0 + d * NW * RPW, in_wave = r % TN;
+            const size_t row = (size_t)(r / TN) * (TN / 2) + (size_t)(in_wave % (TN / 2)) + (in_wave >= TN / 2 ? (size_t)a.gate : 0);
+            req_off_gated[d] = (unsigned)((row * K + (size_t)chunk * 8) * 2);
+        }
+    }
+    constexpr int B_TILE_ROWS = GATED ? BN / 2 : BN;   // rows of (either matrix of) B between two tiles
     const unsigned lds_wave = (unsigned)(unsigned long)(__attribute__((address_space(3))) unsigned char*)smem_raw + (unsigned)wave * 1024u;
 
     // The request stream: the K tile whose requests come next, as base pointers into A and B, and where it sits in its
@@ -153,7 +168,7 @@ __global__ void __launch_bounds__(256) hgemm_f16_big_kernel(HgemmArgs a) {
         int tm, tn;
         tile_of_block(req_vb, total_tiles, tiles_m, band_m, tm, tn);
         req_a_tile = Ag + (size_t)tm * BM * row_bytes;
-        req_b_tile = Bg + (size_t)tn * BN * row_bytes;
+        req_b_tile = Bg + (size_t)tn * B_TILE_ROWS * row_bytes;
         req_w = 0;
         req_k = (int)(((unsigned)tn * rot_tile + (blockIdx.x & 7u) * rot_xcd) % (unsigned)KT);
     };
@@ -182,6 +197,8 @@ __global__ void __launch_bounds__(256) hgemm_f16_big_kernel(HgemmArgs a) {
         constexpr int d = decltype(dd)::value, st = decltype(stage)::value;
         if constexpr (d < A_REQS)
             request_16B_per_lane<st * STAGE_BYTES + d * NW * 1024>(pa, req_off[d], lds_wave);
+        else if constexpr (GATED)
+            request_16B_per_lane<st * STAGE_BYTES + A_BYTES + (d - A_REQS) * NW * 1024>(pb, req_off_gated[d - A_REQS], lds_wave);
         else
             request_16B_per_lane<st * STAGE_BYTES + A_BYTES + (d - A_REQS) * NW * 1024>(pb, req_off[d - A_REQS], lds_wave);
     };
@@ -279,9 +296,9 @@ __global__ void __launch_bounds__(256) hgemm_f16_big_kernel(HgemmArgs a) {
         tile_of_block(vb, total_tiles, tiles_m, band_m, tm, tn);
         const int e_row = lane & 15;
         const int e_col = (lane >> 4) * 4;
-        const int row_base = tm * BM + wm * TM, col_base = tn * BN + wn * TN;
+        const int row_base = tm * BM + wm * TM, col_base = GATED ? tn * (BN / 2) + wn * (TN / 2) : tn * BN + wn * TN;
         constexpr int RS = TN * 2 + 16;
-        constexpr int CH = TN / 8;               // 16-byte chunks per row
+        constexpr int CH = (GATED ? TN / 2 : TN) / 8;   // 16-byte chunks per row of output
         constexpr int RPR = 64 / CH;             // rows per wavefront-wide read
         constexpr int PASSES = 16 / RPR;
         static_assert(64 % CH == 0 && 16 % RPR == 0, "a staged block is read back in whole wavefront-wide passes");
@@ -296,10 +313,27 @@ __global__ void __launch_bounds__(256) hgemm_f16_big_kernel(HgemmArgs a) {
 #pragma unroll
             for (int q = 0; q < PASSES; ++q) {
                 const int r = q * RPR + lane / CH, c = lane % CH;
-                const half8_t v = *reinterpret_cast<const half8_t*>(region + r * RS + c * 16);
                 const int row = row_base + i * 16 + r, col = col_base + c * 8;
-                if (col < N) *reinterpret_cast<half8_t*>(C + (size_t)row * ldc + col) = v;
+                if constexpr (GATED) {
+                    // pairs of 16-byte pieces TN/2 columns apart: out = half(silu(x) * y) of the two rounded projections,
+                    // the arithmetic of the separate gate kernel
+                    const half8_t vx = *reinterpret_cast<const half8_t*>(region + r * RS + c * 16);
+                    const half8_t vy = *reinterpret_cast<const half8_t*>(region + r * RS + TN + c * 16);
+                    half8_t o;
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) {
+                        const float x = (float)vx[e];
+                        o[e] = (half_t)(x * (1.0f / (1.0f + expf(-x))) * (float)vy[e]);
+                    }
+                    *reinterpret_cast<half8_t*>(C + (size_t)row * ldc + col) = o;
+                } else {
+                    const half8_t v = *reinterpret_cast<const half8_t*>(region + r * RS + c * 16);
+                    if (col < N) *reinterpret_cast<half8_t*>(C + (size_t)row * ldc + col) = v;
+                }
             }
+            // one block of accumulators at a time: without this the gate's arithmetic invites the scheduler to pull
+            // every block's accumulators into VGPRs first
+            if constexpr (GATED) __builtin_amdgcn_sched_barrier(0);
         }
         vb += (int)gridDim.x;
         if (vb >= total_tiles) break;
@@ -553,28 +587,32 @@ int launch_hgemm_mid(const void* A, const void* B, void* C, size_t M, size_t N, 
     return TL_OK;
 }
 
-static std::atomic<bool> g_big_attr{false};
+static std::atomic<bool> g_big_attr{false}, g_big_gated_attr{false};
 
 const char* hgemm_big_name() { return "a256x256x64w2x2"; }
 
 // Full contract of the kernel: whole 256x256 tiles, an even number of K tiles of 64, at least four, lane offsets of a
-// tile within 32 bits, C rows that take 16-byte stores.
-bool hgemm_big_applies(const void* A, const void* B, const void* C, size_t M, size_t N, size_t K, size_t ldc) {
+// tile within 32 bits, C rows that take 16-byte stores.  gate != 0: N counts the rows of both matrices in B, C has N / 2
+// columns in whole tiles of 128, and the lane offsets reach the second matrix.
+bool hgemm_big_applies(const void* A, const void* B, const void* C, size_t M, size_t N, size_t K, size_t ldc, size_t gate) {
+    const size_t n_out = gate ? N / 2 : N;
     return M >= 256 && N >= 256 && M % 256 == 0 && N % 256 == 0 && K >= 256 && K % 128 == 0 && K <= ((size_t)1 << 22) &&
-           ldc % 8 == 0 && ldc >= N && aligned16(A) && aligned16(B) && aligned16(C) && M <= 0x7fffffffu && N <= 0x7fffffffu;
+           ldc % 8 == 0 && ldc >= n_out && aligned16(A) && aligned16(B) && aligned16(C) && M <= 0x7fffffffu && N <= 0x7fffffffu &&
+           (gate == 0 || (gate >= n_out && gate <= 0x7fffffffu && (gate + n_out) * K * sizeof(half_t) < ((size_t)1 << 32)));
 }
 
 int launch_hgemm_big(const void* A, const void* B, void* C, size_t M, size_t N, size_t K, size_t ldc, int band, int rot_tile,
-                     int rot_xcd) {
-    TL_REQUIRE(hgemm_big_applies(A, B, C, M, N, K, ldc), "hgemm: %s does not serve this shape", hgemm_big_name());
+                     int rot_xcd, size_t gate) {
+    TL_REQUIRE(hgemm_big_applies(A, B, C, M, N, K, ldc, gate), "hgemm: %s does not serve this shape", hgemm_big_name());
     // A fragments read three iterations ahead, the barrier in front of iteration 13 of 16, a request every fourth MFMA:
     // A_AHEAD 3 .. 6, barriers at 11 .. 13 and request spacings 3 and 4 measured within 1 % of each other
-    void (*const kernel)(HgemmArgs) = hgemm_f16_big_kernel<3, 13, 4>;
+    void (*const kernel)(HgemmArgs) = gate ? hgemm_f16_big_kernel<3, 13, 4, true> : hgemm_f16_big_kernel<3, 13, 4, false>;
     // the two-stage ring and behind it the C staging of the epilogue (four wavefronts x 16 rows x (256 + 16) bytes)
     const size_t lds = (size_t)2 * (256 + 256) * 64 * sizeof(half_t) + (size_t)4 * 16 * (128 * 2 + 16);
-    if (!g_big_attr.load()) {
+    std::atomic<bool>& attr = gate ? g_big_gated_attr : g_big_attr;
+    if (!attr.load()) {
         TL_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-        g_big_attr.store(true);
+        attr.store(true);
     }
     HgemmArgs a{};
     a.A = (const half_t*)A;
@@ -585,11 +623,12 @@ int launch_hgemm_big(const void* A, const void* B, void* C, size_t M, size_t N, 
     a.K = (int)K;
     a.ldc = (int)ldc;
     a.tiles_m = (int)(M / 256);
-    a.tiles_n = (int)(N / 256);
+    a.tiles_n = (int)(N / 256);   // a gated tile covers 128 output columns: N / 2 / 128
     a.kt_per_split = 0x7fffffff;
     a.band_m = band > 0 ? band : 8;
     a.rot_tile = rot_tile;
     a.rot_xcd = rot_xcd;
+    a.gate = (int)gate;
     const size_t nblocks = (size_t)a.tiles_m * a.tiles_n;
     TL_REQUIRE(nblocks <= 0x7fffffffu, "hgemm: too many tiles");
     // persistent: one workgroup per CU walks tiles blockIdx.x, + gridDim.x, ...

@@ -59,9 +59,10 @@ __device__ __forceinline__ void tile_of_block(int bid, int nblocks, int tiles_m,
 // The kernel of hgemm_agpr.hip (256x256 tiles, one wavefront per SIMD, accumulators in AGPRs).  band / rot_*: as in
 // HgemmArgs.
 const char* hgemm_big_name();
-bool hgemm_big_applies(const void* A, const void* B, const void* C, size_t M, size_t N, size_t K, size_t ldc);
+// gate: 0, or HgemmArgs::gate of a gated launch (N then counts the rows of both matrices in B, C has N / 2 columns).
+bool hgemm_big_applies(const void* A, const void* B, const void* C, size_t M, size_t N, size_t K, size_t ldc, size_t gate = 0);
 int launch_hgemm_big(const void* A, const void* B, void* C, size_t M, size_t N, size_t K, size_t ldc, int band, int rot_tile,
-                     int rot_xcd);
+                     int rot_xcd, size_t gate = 0);
 // and its 256x128 sibling (three-stage ring, one C tile per workgroup)
 const char* hgemm_mid_name();
 bool hgemm_mid_applies(const void* A, const void* B, const void* C, size_t M, size_t N, size_t K, size_t ldc);

@@ -400,7 +400,7 @@ def test_hgemm_silu_mul_equals_two_steps(dev, shape):
     a = X.double() @ W13[:hidden].double().T
     b = X.double() @ W13[hidden:].double().T
     ref = (a.half().double() / (1.0 + torch.exp(-a.half().double())) * b.half().double())
-    assert_close_f16(got.cpu().numpy(), ref.cpu().numpy().astype(np.float16), RTOL, 2e-3, f"gated {shape}")
+    assert_close_f16(got.cpu().numpy(), ref.cpu().numpy().astype(np.float16), RTOL, ATOL, f"gated {shape}")
 
 
 @pytest.mark.parametrize("M", [128, 512, 2048])
@@ -411,6 +411,8 @@ def test_hgemm_silu_mul_against_the_oracle(dev, oracle, M):
     X = synth.normal_f16(7850 + M, (M, K), 1.0)
     W13 = synth.normal_f16(7851, (2 * hidden, K), 0.02)
     got = dev.hgemm_silu_mul(dev.from_numpy(X), dev.from_numpy(W13)).cpu().numpy()
+    if M >= 512:   # whole 256-row tiles: the gated build of the AGPR kernel serves (at least the last columns of) these
+        assert dev.hgemm_last_plan()[0] == "a256x256x64w2x2"
     rng = np.random.default_rng(M)
     rows = np.unique(np.concatenate([[0, M - 1], rng.integers(0, M, 6)]))
     want = oracle.silu_mul(oracle.matmul2d(X[rows], W13[:hidden]), oracle.matmul2d(X[rows], W13[hidden:]))

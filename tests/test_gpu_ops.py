@@ -380,6 +380,32 @@ def test_hgemm_prefill_rope_qkv_vt_equals_separate_calls(dev, S, H, D, K):
     assert torch.equal(q2, q1) and torch.equal(k2, k1) and torch.equal(v2, v1) and torch.equal(vT2, vT1), f"splits {split}"
 
 
+def test_hgemm_prefill_rope_qkv_vt_rejects_before_it_writes(dev):
+    """Arguments of the second step (the rotation) are checked before the projection is launched: a call with an ldv
+    that does not cover the tokens, or a missing output, fails and leaves the qkv buffer as it was."""
+    TL_OK = 0
+    S, H, D, K = 128, 8, 64, 512
+    dim = H * D
+    X = dev.from_numpy(synth.normal_f16(180, (S, K), 1.0))
+    W = dev.from_numpy(synth.normal_f16(181, (3 * dim, K), 0.02))
+    table = dev.rope_table(S, D)
+    qkv = torch.full((S, 3 * dim), 7.0, dtype=torch.float16, device="cuda")
+    q, kc, vc = dev.empty(H, S, D), dev.empty(S, H, D), dev.empty(S, H, D)
+    vT = dev.empty(H, D, S)
+    p = lambda t: t.data_ptr()
+    lib = dev.lib
+    rc = lib.tl_hgemm_prefill_rope_qkv_vt_f16(p(X), p(W), p(qkv), p(q), p(kc), p(vc), p(table), p(vT), 64, S, H, D, K)     # ldv < S
+    assert rc != TL_OK
+    rc = lib.tl_hgemm_prefill_rope_qkv_vt_f16(p(X), p(W), p(qkv), p(q), p(kc), p(vc), p(table), None, S, S, H, D, K)      # no vT
+    assert rc != TL_OK
+    rc = lib.tl_hgemm_prefill_rope_qkv_vt_f16(p(X), p(W), p(qkv), p(q) + 2, p(kc), p(vc), p(table), p(vT), S, S, H, D, K)  # unaligned q
+    assert rc != TL_OK
+    torch.cuda.synchronize()
+    assert bool((qkv == 7.0).all())
+    rc = lib.tl_hgemm_prefill_rope_qkv_vt_f16(p(X), p(W), p(qkv), p(q), p(kc), p(vc), p(table), p(vT), S, S, H, D, K)
+    assert rc == TL_OK
+
+
 @pytest.mark.parametrize("S", [128, 512, 33])
 def test_hgemm_prefill_rope_qkv_vt_against_the_oracle(dev, oracle, S):
     """The fused projection + rotation entry against the CPU restatement directly: oracle.matmul2d of sampled token rows
