@@ -45,7 +45,7 @@ HGEMM_SHAPES = [(2048, 4096, 4096), (2048, 11008, 4096), (2048, 32000, 4096), (2
 # size (FETCH_SIZE x 1.9997 KiB, WRITE_SIZE x 1.0000 KiB); algorithmic bytes per launch are 119,050,624.
 # Counters cannot be read inside this process: the figure comes from the profile named beside it and is
 # reported with that source, not re-measured by a bench run.
-GEMV_TRAFFIC_BYTES_PER_LAUNCH = 119_423_152
+GEMV_TRAFFIC_BYTES_PER_LAUNCH = 119_420_779
 GEMV_TRAFFIC_SOURCE = "profiles/gemv_decode_sweep_hbm_traffic.txt (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of this command)"
 
 
@@ -54,7 +54,7 @@ def parse_args():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", choices=["gemv", "hgemm", "decode", "gemv_timeline", "gemv_grid"], default="gemv")
+    ap.add_argument("--workload", choices=["gemv", "hgemm", "decode", "gemv_timeline", "gemv_grid", "hgemm_timeline"], default="gemv")
     ap.add_argument("--rows", default="2048",
                     help="--workload hgemm: row counts M of the prefill shapes that form the timed step, comma separated, "
                          "from 16 (the four projections of a 16-token prompt), 128, 512, 2048")
@@ -278,6 +278,62 @@ def gemv_timeline(dev, randn, torch, launches: int):
     }
 
 
+def hgemm_timeline(dev, randn, torch, synth, launches: int):
+    """Where the time of a launch of the AGPR GEMM kernels goes, for the four M = 2048 prefill shapes and 512x32000x4096:
+    every workgroup stamps the GPU's constant 100 MHz counter at its first instruction and after its last store
+    (tl_set_hgemm_stamps).  `launches` back-to-back calls of tl_matmul2d_f16 per shape, W rotating over >= 600 MB.
+    Per shape, medians over the launches, microseconds after the first workgroup's start: the last workgroup's start,
+    mean / shortest / longest workgroup, 10 / 50 / 90 / 100 % of the workgroups done, and the period to the next
+    launch's first start (what lies between the window and the period is the launch boundary).  A call that goes out
+    as two launches (whole rounds of 256x256 tiles, then the remaining columns) reports the second one's workgroups
+    where both wrote a stamp slot and is marked."""
+    import numpy as np
+    launches = max(6, min(launches, 40))
+    cap = 2 * 4096
+    out = {}
+    for (M, N, K) in [s for s in HGEMM_SHAPES if s[0] == 2048] + [(512, 32000, 4096)]:
+        A = randn((M, K), 1.0)
+        nb = max(2, -(-600_000_000 // (N * K * 2)))
+        Bs = [randn((N, K), 0.02) for _ in range(nb)]
+        C = torch.empty((M, N), device="cuda", dtype=torch.float16)
+        for i in range(4):
+            dev.matmul2d(A, Bs[i % nb], C)
+        stamps = torch.zeros((launches, cap), device="cuda", dtype=torch.int64)
+        torch.cuda.synchronize()
+        try:
+            for i in range(launches):
+                dev.lib.tl_set_hgemm_stamps(stamps[i].data_ptr(), cap)
+                dev.matmul2d(A, Bs[i % nb], C)
+        finally:
+            dev.lib.tl_set_hgemm_stamps(None, 0)
+        torch.cuda.synchronize()
+        plan = dev.hgemm_last_plan()
+        st = stamps.cpu().numpy().astype(np.float64) * 0.01   # us
+        n = int((st[0] != 0).sum() // 2)
+        if n == 0:
+            out[f"{M}x{N}x{K}"] = {"kernel": plan[0], "note": "no stamped kernel served this shape"}
+            continue
+        t = st[:, :2 * n].reshape(launches, n, 2)
+        first = t[:, :, 0].min(axis=1)
+        start, end = t[:, :, 0] - first[:, None], t[:, :, 1] - first[:, None]
+        dur = end - start
+        ends = np.sort(end, axis=1)
+        q = lambda f: round(float(np.median(ends[:, min(n - 1, int(f * n))])), 1)
+        window = ends[:, -1]
+        flops = synth.gemm_flops(M, N, K)
+        period = float(np.median(np.diff(first)))
+        out[f"{M}x{N}x{K}"] = {
+            "kernel": plan[0], "workgroups_stamped": n, "two_launches": bool(np.median(start.max(axis=1)) > 5.0),
+            "last_start_us": round(float(np.median(start.max(axis=1))), 1),
+            "workgroup_us": {"mean": round(float(np.median(dur.mean(axis=1))), 1), "min": round(float(np.median(dur.min(axis=1))), 1),
+                             "max": round(float(np.median(dur.max(axis=1))), 1)},
+            "workgroups_done_us": {"10%": q(0.10), "50%": q(0.50), "90%": q(0.90), "100%": round(float(np.median(window)), 1)},
+            "period_us": round(period, 1), "outside_window_us": round(float(np.median(np.diff(first) - window[:-1])), 1),
+            "TFLOP/s_at_period": round(flops / period / 1e6, 1),
+        }
+    return {"metric": "time line of the AGPR fp16 GEMM kernels (workgroup time stamps)", "launches": launches, "shapes": out}
+
+
 def gemv_grid_experiments(dev, randn, torch, synth):
     """The plain streaming GEMV under capped, persistent grids and with four rows per wavefront pass, W from HBM:
     4096<-4096 and 12288<-4096, every configuration timed over 200 launches on > 1 GB of rotating matrices."""
@@ -368,6 +424,9 @@ def main():
 
     if args.workload == "gemv_timeline":
         print(json.dumps(gemv_timeline(dev, randn, torch, args.steps)))
+        return
+    if args.workload == "hgemm_timeline":
+        print(json.dumps(hgemm_timeline(dev, randn, torch, synth, args.steps)))
         return
     if args.workload == "gemv_grid":
         print(json.dumps(gemv_grid_experiments(dev, randn, torch, synth)))

@@ -139,6 +139,11 @@ int tl_hgemm_last_plan(int* variant, int* splits);
  * a256x256x64w2x2, a256x128x64w2x2) wherever whole tiles of theirs cover the problem, -1 = never (the ring kernels with
  * 32x32x16 MFMAs serve every shape, as they do for partly filled tiles). */
 int tl_set_hgemm_agpr_kernels(int mode);
+/* Inspection hook (no reference counterpart): while `stamps` is not NULL, every launch of those two kernels with at most
+ * capacity / 2 workgroups writes stamps[2 * w] / stamps[2 * w + 1] = the GPU's constant 100 MHz counter at workgroup w's
+ * first instruction and after its last store (device memory, `capacity` 64-bit words).  bench.py --workload
+ * hgemm_timeline turns them into the time line of a launch.  NULL switches it off. */
+int tl_set_hgemm_stamps(void* stamps, size_t capacity);
 /* Tuning hook: where the fp32 partial sums of a split-K GEMM are added up.  0 = automatic and 2 = by a second kernel
  * (the default: measured faster on every split shape); 1 = inside the GEMM launch, by the workgroup that finishes a
  * C tile's last split (one counter per tile in the library's scratch, zero between launches), whenever C takes 8-byte

@@ -68,6 +68,7 @@ _PROTOS = {
     "tl_set_hgemm_splits": (_i, [_i]),
     "tl_set_hgemm_splitk_merge": (_i, [_i]),
     "tl_set_hgemm_agpr_kernels": (_i, [_i]),
+    "tl_set_hgemm_stamps": (_i, [_vp, _sz]),
     "tl_hgemm_last_split_in_launch": (_i, []),
     "tl_hgemm_last_plan": (_i, [_c.POINTER(_c.c_int), _c.POINTER(_c.c_int)]),
     "tl_set_hgemm_k_rotation": (_i, [_i, _i]),

@@ -1280,6 +1280,11 @@ int tl_set_hgemm_agpr_kernels(int mode) {
     return TL_OK;
 }
 
+int tl_set_hgemm_stamps(void* stamps, size_t capacity) {
+    tl::hgemm_agpr_set_stamps(stamps, capacity);
+    return TL_OK;
+}
+
 int tl_set_hgemm_splitk_merge(int mode) {
     TL_REQUIRE(mode >= 0 && mode <= 2, "tl_set_hgemm_splitk_merge: %d out of range [0,2]", mode);
     tl::g_splitk_merge_mode = mode;

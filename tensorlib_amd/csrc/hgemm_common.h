@@ -29,6 +29,9 @@ struct HgemmArgs {
     // Gated launches (kernels built with MODE 2): B holds two matrices `gate` rows apart, N counts the rows of both
     // (2 x the output columns), and C[m][n] = silu(A[m,:].B[n,:]) * (A[m,:].B[gate + n,:]) for n < N / 2.
     int gate;
+    // Inspection (the kernels of hgemm_agpr.hip): when not null, stamps[2 * workgroup] / [2 * workgroup + 1] receive the
+    // constant 100 MHz counter (s_memrealtime) at the workgroup's first instruction and after its last store.
+    unsigned long long* stamps;
 };
 
 // Map the linear workgroup id to a tile so that workgroups resident on one XCD (ids
@@ -63,6 +66,9 @@ const char* hgemm_big_name();
 bool hgemm_big_applies(const void* A, const void* B, const void* C, size_t M, size_t N, size_t K, size_t ldc, size_t gate = 0);
 int launch_hgemm_big(const void* A, const void* B, void* C, size_t M, size_t N, size_t K, size_t ldc, int band, int rot_tile,
                      int rot_xcd, size_t gate = 0);
+// Inspection: the following launches of both kernels write 2 x workgroups time stamps (HgemmArgs::stamps) into buf when it
+// holds that many 64-bit words; null switches it off.
+void hgemm_agpr_set_stamps(void* buf, size_t capacity);
 // and its 256x128 sibling (three-stage ring, one C tile per workgroup)
 const char* hgemm_mid_name();
 bool hgemm_mid_applies(const void* A, const void* B, const void* C, size_t M, size_t N, size_t K, size_t ldc);

@@ -868,6 +868,37 @@ def test_hgemm_agpr_kernels_can_be_switched_off(dev):
         dev.lib.tl_set_hgemm_agpr_kernels(0)
 
 
+def test_hgemm_agpr_kernels_write_time_stamps_on_request(dev):
+    """tl_set_hgemm_stamps: both AGPR kernels stamp start and end of every workgroup (end after start, all within a
+    second of each other), leave the result alone, write nothing when the buffer is too small or switched off."""
+    names = dev.hgemm_variants()
+    A = dev.from_numpy(synth.small_ints_f16(9600, (512, 512), -2, 2))
+    B = dev.from_numpy(synth.small_ints_f16(9601, (1024, 512), -2, 2))
+    want = A.double() @ B.double().T
+    try:
+        for name, wgs in (("a256x256x64w2x2", 2 * 4), ("a256x128x64w2x2", 2 * 8)):
+            dev.set_hgemm_variant(names.index(name))
+            stamps = torch.zeros(2 * wgs + 6, dtype=torch.int64, device="cuda")
+            dev.lib.tl_set_hgemm_stamps(stamps.data_ptr(), 2 * wgs + 6)
+            C = dev.hgemm(A, B)
+            assert dev.hgemm_last_plan()[0] == name and torch.equal(C.double(), want)
+            t = stamps.cpu().numpy()
+            assert (t[:2 * wgs] != 0).all() and (t[2 * wgs:] == 0).all(), name
+            t = t[:2 * wgs].reshape(wgs, 2)
+            assert (t[:, 1] > t[:, 0]).all() and t.max() - t.min() < 100_000_000, name
+            small = torch.zeros(2 * wgs, dtype=torch.int64, device="cuda")
+            dev.lib.tl_set_hgemm_stamps(small.data_ptr(), 2 * wgs - 2)     # does not hold every workgroup: untouched
+            C = dev.hgemm(A, B)
+            assert torch.equal(C.double(), want) and not bool(small.any())
+            dev.lib.tl_set_hgemm_stamps(None, 0)
+            stamps.zero_()
+            dev.hgemm(A, B)
+            assert not bool(stamps.any())
+    finally:
+        dev.lib.tl_set_hgemm_stamps(None, 0)
+        dev.set_hgemm_variant(0)
+
+
 def test_hgemm_256x256_agpr_kernel_falls_back_on_partial_tiles(dev, oracle):
     """Rows or columns that do not fill whole 256x256 tiles, a K that is not an even number of tiles: the forced variant
     hands the call to the ring kernel."""
