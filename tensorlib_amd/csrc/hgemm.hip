@@ -1047,7 +1047,10 @@ static int launch_hgemm_cols(const void* A, const void* B, void* C, size_t M, si
         const int forced_band = g_forced_band.load();
         const int rt = g_forced_rot_tile.load(), rx = g_forced_rot_xcd.load();
         const bool mid = g_variants[vi].stages == -2;
-        const int band = forced_band > 0 ? forced_band : 8, rot_tile = rt >= 0 ? rt : 0, rot_xcd = rx >= 0 ? rx : (int)(K / 64 / 8);
+        // bands of four rows of tiles: the 32 tiles an XCD runs at a time then cover 4 panels of A and 8 of B (measured
+        // against bands of 8, same box: 2048x32000x4096 392 -> 378 us, 2048x22016x4096 286 -> 275, 2048x4096x11008 147 -> 142,
+        // 8192x8192x8192 equal)
+        const int band = forced_band > 0 ? forced_band : 4, rot_tile = rt >= 0 ? rt : 0, rot_xcd = rx >= 0 ? rx : (int)(K / 64 / 8);
         if (batch == 1 && (mid ? gate == 0 && hgemm_mid_applies(A, B, C, M, N, K, ldc) : hgemm_big_applies(A, B, C, M, N, K, ldc, gate))) {
             g_last_variant = vi;
             g_last_splits = 1;
