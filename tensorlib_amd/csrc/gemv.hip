@@ -100,9 +100,24 @@ struct GemvArgs {
     unsigned long long* stamps;
 };
 
+// The kernels take GemvArgs' fields as separate scalar parameters, not the struct: the first 16 dwords of scalar kernel
+// arguments (x, W, y, N, K8, the block count and the batch strides) are then preloaded into SGPRs when a wavefront is
+// launched (-mllvm -amdgpu-kernarg-preload-count=16; a struct passed by value is not), and a wavefront's first address
+// does not wait for a scalar load from the argument buffer.  On firmware without the feature the same code runs
+// through the compiler's compatibility prologue, which loads them.
+#define TL_GEMV_PARAMS                                                                                                 \
+    const half8_t *p_x, const half8_t *p_W, half_t *p_y, int p_N, int p_K8, int p_blocks, long p_sx8, long p_sw8,     \
+        long p_sy, const half8_t *p_x2, const half8_t *p_g, half8_t *p_sum_out, float p_eps, unsigned long long *p_stamps
+#define TL_GEMV_ARGS_FROM_PARAMS \
+    const GemvArgs a { p_x, p_W, p_y, p_N, p_K8, p_blocks, p_sx8, p_sw8, p_sy, p_x2, p_g, p_sum_out, p_eps, p_stamps }
+#define TL_GEMV_PASS(a) \
+    (a).x, (a).W, (a).y, (a).N, (a).K8, (a).num_row_blocks, (a).sx8, (a).sw8, (a).sy, (a).x2, (a).g, (a).sum_out, (a).eps, (a).stamps
+typedef void (*GemvKernel)(TL_GEMV_PARAMS);
+
 // One wavefront per row group.  Dynamic LDS: K8 chunks of x (+ partial sums when KSPLIT > 1).
 template <int WAVES, int ROWS, int UNROLL, int KSPLIT, bool NT>
-__global__ void __launch_bounds__(WAVES * 64) gemv_f16_wave_kernel(GemvArgs a) {
+__global__ void __launch_bounds__(WAVES * 64) gemv_f16_wave_kernel(TL_GEMV_PARAMS) {
+    TL_GEMV_ARGS_FROM_PARAMS;
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
     half8_t* xs = reinterpret_cast<half8_t*>(smem_raw);
 
@@ -210,7 +225,8 @@ __global__ void __launch_bounds__(WAVES * 64) gemv_f16_wave_kernel(GemvArgs a) {
 // STAMP: measurement build (tl_gemv_f16_stamped): thread 0 of every workgroup records the time at its first
 // instruction and after the workgroup's last store; otherwise the same instructions.
 template <int WAVES, int ROWS, int UNROLL, int KSPLIT, int XMODE, bool STAMP = false>
-__global__ void __launch_bounds__(WAVES * 64) gemv_f16_stream_kernel(GemvArgs a) {
+__global__ void __launch_bounds__(WAVES * 64) gemv_f16_stream_kernel(TL_GEMV_PARAMS) {
+    TL_GEMV_ARGS_FROM_PARAMS;
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
     half8_t* xs = reinterpret_cast<half8_t*>(smem_raw);
 
@@ -378,7 +394,8 @@ __global__ void __launch_bounds__(WAVES * 64) gemv_f16_stream_kernel(GemvArgs a)
 // Short rows (K8 < 64 chunks): LPR lanes per row, 64/LPR rows per wavefront pass; x read
 // straight from global memory (it is at most 1 KiB).  Serves attention's q.K^T (K = 128).
 template <int LPR>
-__global__ void __launch_bounds__(256) gemv_f16_short_kernel(GemvArgs a) {
+__global__ void __launch_bounds__(256) gemv_f16_short_kernel(TL_GEMV_PARAMS) {
+    TL_GEMV_ARGS_FROM_PARAMS;
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = tid >> 6;
@@ -427,7 +444,7 @@ struct GemvVariant {
     const char* name;
     int waves, rows, unroll, ksplit;
     int xmode;  // -1: looping kernel (any K), 0/1: single-tile streaming kernel
-    void (*kernel)(GemvArgs);
+    GemvKernel kernel;
 };
 
 #define TL_LOOP(W_, R_, U_, S_, NT_) \
@@ -541,11 +558,11 @@ int launch_gemv(const void* x, const void* W, void* y, size_t N, size_t K, size_
         if (blocks > cap) blocks = cap;
         dim3 grid(blocks, (unsigned)batch);
         if (lpr == 32)
-            hipLaunchKernelGGL(gemv_f16_short_kernel<32>, grid, dim3(256), 0, st, a);
+            hipLaunchKernelGGL(gemv_f16_short_kernel<32>, grid, dim3(256), 0, st, TL_GEMV_PASS(a));
         else if (lpr == 16)
-            hipLaunchKernelGGL(gemv_f16_short_kernel<16>, grid, dim3(256), 0, st, a);
+            hipLaunchKernelGGL(gemv_f16_short_kernel<16>, grid, dim3(256), 0, st, TL_GEMV_PASS(a));
         else
-            hipLaunchKernelGGL(gemv_f16_short_kernel<8>, grid, dim3(256), 0, st, a);
+            hipLaunchKernelGGL(gemv_f16_short_kernel<8>, grid, dim3(256), 0, st, TL_GEMV_PASS(a));
         TL_CHECK_LAUNCH("gemv_f16_short_kernel");
         return TL_OK;
     }
@@ -606,7 +623,7 @@ int launch_gemv(const void* x, const void* W, void* y, size_t N, size_t K, size_
     long cap = (long)dev.cu_count * wpc / v.waves;
     if (cap < 1) cap = 1;
     if (blocks > cap) blocks = (int)cap;
-    hipLaunchKernelGGL(v.kernel, dim3(blocks, (unsigned)batch), dim3(v.waves * 64), lds, st, a);
+    hipLaunchKernelGGL(v.kernel, dim3(blocks, (unsigned)batch), dim3(v.waves * 64), lds, st, TL_GEMV_PASS(a));
     TL_CHECK_LAUNCH(v.name);
     return TL_OK;
 }
@@ -661,7 +678,7 @@ extern "C" int tl_gemv_f16_stamped(const void* x, const void* W, void* y, size_t
     *workgroups = a.num_row_blocks;
     const size_t lds = (size_t)2 * (WAVES / KSPLIT) * KSPLIT * ROWS * 4;
     hipLaunchKernelGGL((tl::gemv_f16_stream_kernel<WAVES, ROWS, 2, KSPLIT, 1, true>), dim3(a.num_row_blocks), dim3(WAVES * 64), lds,
-                       tl::stream(), a);
+                       tl::stream(), TL_GEMV_PASS(a));
     TL_CHECK_LAUNCH("gemv_f16_stream_kernel<stamped>");
     return TL_OK;
 }

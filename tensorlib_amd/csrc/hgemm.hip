@@ -29,7 +29,8 @@ namespace tl {
 constexpr int kPad = 8;  // halves of padding per LDS row
 
 template <int BM, int BN, int BK, int WM, int WN>
-__global__ void __launch_bounds__(WM* WN * 64) hgemm_f16_mfma_kernel(HgemmArgs a) {
+__global__ void __launch_bounds__(WM* WN * 64) hgemm_f16_mfma_kernel(TL_HGEMM_PARAMS) {
+    TL_HGEMM_ARGS_FROM_PARAMS;
     constexpr int THREADS = WM * WN * 64;
     constexpr int LDS_ROW = BK + kPad;          // halves
     constexpr int CPR = BK / 8;                 // 16-byte chunks per tile row
@@ -175,7 +176,8 @@ __global__ void __launch_bounds__(WM* WN * 64) hgemm_f16_mfma_kernel(HgemmArgs a
 //         first matrix followed by the TN/2 rows of the second that pair with them, so a wavefront finds both factors
 //         of an output in the 32 x TN block it stages through LDS anyway; the tile then covers BN/2 output columns.
 template <int BM, int BN, int BK, int WM, int WN, int STAGES, int MODE>
-__global__ void __launch_bounds__(WM* WN * 64) hgemm_f16_dlds_kernel(HgemmArgs a) {
+__global__ void __launch_bounds__(WM* WN * 64) hgemm_f16_dlds_kernel(TL_HGEMM_PARAMS) {
+    TL_HGEMM_ARGS_FROM_PARAMS;
     constexpr int NW = WM * WN;
     constexpr int RB = BK * 2;                 // bytes per tile row
     constexpr int CPR = BK / 8;                // 16-byte chunks per tile row
@@ -735,9 +737,9 @@ struct HgemmVariant {
     const char* name;
     int bm, bn, bk, threads;
     int stages;  // 0: register-staged kernel (any K % 8 == 0); >= 2: direct-to-LDS ring (K % bk == 0)
-    void (*kernel)(HgemmArgs);
+    HgemmKernel kernel;
     bool persistent;  // the kernel walks tiles blockIdx.x, + gridDim.x, ... (same predicate as PERSIST in the kernel)
-    void (*gated_kernel)(HgemmArgs);  // the same kernel with the SwiGLU gate in its epilogue (pipelined variants), else null
+    HgemmKernel gated_kernel;  // the same kernel with the SwiGLU gate in its epilogue (pipelined variants), else null
 };
 
 #define TL_HGEMM_VARIANT(BM, BN, BK, WM, WN) \
@@ -1066,7 +1068,7 @@ static int launch_hgemm_cols(const void* A, const void* B, void* C, size_t M, si
     if (g_variants[vi].stages > 0 && K > ((size_t)1 << 22)) vi = 1;
     const HgemmVariant& v = g_variants[vi];
     const size_t lds = lds_bytes(v);
-    void (*const kernel)(HgemmArgs) = gate ? v.gated_kernel : v.kernel;
+    const HgemmKernel kernel = gate ? v.gated_kernel : v.kernel;
     if (gate) {
         // what hgemm_gated_applies checks, once more where a violation would fault: the pipelined kernel, a C the
         // staged epilogue can store to in 16-byte pieces, and 32-bit lane offsets that reach both matrices
@@ -1166,7 +1168,7 @@ static int launch_hgemm_cols(const void* A, const void* B, void* C, size_t M, si
         if (rt >= 0) a.rot_tile = rt;
         if (rx >= 0) a.rot_xcd = rx;
     }
-    hipLaunchKernelGGL(kernel, dim3((unsigned)grid_x, (unsigned)batch, (unsigned)splits), dim3(v.threads), lds, st, a);
+    hipLaunchKernelGGL(kernel, dim3((unsigned)grid_x, (unsigned)batch, (unsigned)splits), dim3(v.threads), lds, st, TL_HGEMM_PASS(a));
     TL_CHECK_LAUNCH(v.name);
     if (splits > 1 && partials_out && splits_out) {
         // the caller folds the second pass of split-K into its own kernel

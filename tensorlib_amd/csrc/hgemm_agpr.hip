@@ -88,7 +88,8 @@ __device__ __forceinline__ void request_16B_per_lane(const void* uniform_base, u
 // then holds, per wavefront column, 64 rows of the first matrix followed by the 64 rows of the second one that pair
 // with them, and covers 128 columns of C; the host passes tiles_n and ldc in output columns.
 template <int A_AHEAD, int BAR_IT, int D_STEP, bool GATED>
-__global__ void __launch_bounds__(256) hgemm_f16_big_kernel(HgemmArgs a) {
+__global__ void __launch_bounds__(256) hgemm_f16_big_kernel(TL_HGEMM_PARAMS) {
+    TL_HGEMM_ARGS_FROM_PARAMS;
     constexpr int BM = 256, BN = 256, BK = 64, WN = 2, NW = 4;
     constexpr int RB = BK * 2;                 // bytes per tile row
     constexpr int CPR = BK / 8;                // 16-byte chunks per tile row
@@ -358,7 +359,8 @@ __global__ void __launch_bounds__(256) hgemm_f16_big_kernel(HgemmArgs a) {
                  "+a"(acc[i + 1][1]), "+a"(acc[i + 1][2]), "+a"(acc[i + 1][3]))
 
 template <int A_AHEAD, int BAR_IT, int D_STEP>
-__global__ void __launch_bounds__(256) hgemm_f16_mid_kernel(HgemmArgs a) {
+__global__ void __launch_bounds__(256) hgemm_f16_mid_kernel(TL_HGEMM_PARAMS) {
+    TL_HGEMM_ARGS_FROM_PARAMS;
     constexpr int BM = 256, BN = 128, BK = 64, WN = 2, NW = 4, STAGES = 3;
     constexpr int RB = BK * 2;
     constexpr int CPR = BK / 8;
@@ -578,7 +580,7 @@ bool hgemm_mid_applies(const void* A, const void* B, const void* C, size_t M, si
 int launch_hgemm_mid(const void* A, const void* B, void* C, size_t M, size_t N, size_t K, size_t ldc, int band, int rot_tile,
                      int rot_xcd) {
     TL_REQUIRE(hgemm_mid_applies(A, B, C, M, N, K, ldc), "hgemm: %s does not serve this shape", hgemm_mid_name());
-    void (*const kernel)(HgemmArgs) = hgemm_f16_mid_kernel<3, 13, 4>;
+    const HgemmKernel kernel = hgemm_f16_mid_kernel<3, 13, 4>;
     // the three-stage ring and behind it the C staging of the epilogue (four wavefronts x 16 rows x (128 + 16) bytes)
     const size_t lds = (size_t)3 * (256 + 128) * 64 * sizeof(half_t) + (size_t)4 * 16 * (64 * 2 + 16);
     if (!g_mid_attr.load()) {
@@ -602,7 +604,7 @@ int launch_hgemm_mid(const void* A, const void* B, void* C, size_t M, size_t N, 
     const size_t nblocks = (size_t)a.tiles_m * a.tiles_n;
     TL_REQUIRE(nblocks <= 0x7fffffffu, "hgemm: too many tiles");
     a.stamps = stamps_for(nblocks);
-    hipLaunchKernelGGL(kernel, dim3((unsigned)nblocks), dim3(256), lds, stream(), a);
+    hipLaunchKernelGGL(kernel, dim3((unsigned)nblocks), dim3(256), lds, stream(), TL_HGEMM_PASS(a));
     TL_CHECK_LAUNCH(hgemm_mid_name());
     return TL_OK;
 }
@@ -626,7 +628,7 @@ int launch_hgemm_big(const void* A, const void* B, void* C, size_t M, size_t N, 
     TL_REQUIRE(hgemm_big_applies(A, B, C, M, N, K, ldc, gate), "hgemm: %s does not serve this shape", hgemm_big_name());
     // A fragments read three iterations ahead, the barrier in front of iteration 13 of 16, a request every fourth MFMA:
     // A_AHEAD 3 .. 6, barriers at 11 .. 13 and request spacings 3 and 4 measured within 1 % of each other
-    void (*const kernel)(HgemmArgs) = gate ? hgemm_f16_big_kernel<3, 13, 4, true> : hgemm_f16_big_kernel<3, 13, 4, false>;
+    const HgemmKernel kernel = gate ? hgemm_f16_big_kernel<3, 13, 4, true> : hgemm_f16_big_kernel<3, 13, 4, false>;
     // the two-stage ring and behind it the C staging of the epilogue (four wavefronts x 16 rows x (256 + 16) bytes)
     const size_t lds = (size_t)2 * (256 + 256) * 64 * sizeof(half_t) + (size_t)4 * 16 * (128 * 2 + 16);
     std::atomic<bool>& attr = gate ? g_big_gated_attr : g_big_attr;
@@ -656,7 +658,7 @@ int launch_hgemm_big(const void* A, const void* B, void* C, size_t M, size_t N, 
     const size_t cus = (size_t)device_info().cu_count;
     if (cus > 0 && grid > cus) grid = cus;
     a.stamps = stamps_for(grid);
-    hipLaunchKernelGGL(kernel, dim3((unsigned)grid), dim3(256), lds, stream(), a);
+    hipLaunchKernelGGL(kernel, dim3((unsigned)grid), dim3(256), lds, stream(), TL_HGEMM_PASS(a));
     TL_CHECK_LAUNCH(hgemm_big_name());
     return TL_OK;
 }

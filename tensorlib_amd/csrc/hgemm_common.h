@@ -34,6 +34,24 @@ struct HgemmArgs {
     unsigned long long* stamps;
 };
 
+// The GEMM kernels take the fields of HgemmArgs as separate scalar parameters: the first 16 dwords of scalar kernel
+// arguments (the three pointers, M, N, K, ldc, the tile counts and two strides) are preloaded into SGPRs when a wavefront
+// is launched (-mllvm -amdgpu-kernarg-preload-count=16), which a struct passed by value is not, so a workgroup's first
+// requests do not wait for a scalar load from the argument buffer.
+#define TL_HGEMM_PARAMS                                                                                                   \
+    const half_t *p_A, const half_t *p_B, half_t *p_C, int p_M, int p_N, int p_K, int p_ldc, int p_tiles_m, int p_tiles_n, \
+        long p_sa, long p_sb, long p_sc, int p_kt_per_split, float *p_partial, unsigned *p_tickets, int p_rot_tile,        \
+        int p_rot_xcd, int p_band_m, int p_gate, unsigned long long *p_stamps
+#define TL_HGEMM_ARGS_FROM_PARAMS                                                                                          \
+    const HgemmArgs a {                                                                                                    \
+        p_A, p_B, p_C, p_M, p_N, p_K, p_ldc, p_tiles_m, p_tiles_n, p_sa, p_sb, p_sc, p_kt_per_split, p_partial, p_tickets, \
+            p_rot_tile, p_rot_xcd, p_band_m, p_gate, p_stamps                                                              \
+    }
+#define TL_HGEMM_PASS(a)                                                                                                  \
+    (a).A, (a).B, (a).C, (a).M, (a).N, (a).K, (a).ldc, (a).tiles_m, (a).tiles_n, (a).sa, (a).sb, (a).sc, (a).kt_per_split, \
+        (a).partial, (a).tickets, (a).rot_tile, (a).rot_xcd, (a).band_m, (a).gate, (a).stamps
+typedef void (*HgemmKernel)(TL_HGEMM_PARAMS);
+
 // Map the linear workgroup id to a tile so that workgroups resident on one XCD (ids
 // congruent mod 8 are dispatched to the same XCD) work on neighbouring tiles: XCD x takes a contiguous run of
 // tile numbers, and tiles are numbered down a band of `band` rows of tiles, column after column, band after

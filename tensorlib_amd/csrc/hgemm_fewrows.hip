@@ -58,7 +58,10 @@ constexpr int fewrows_lds_bytes() { return kFrRingBytes + 2 * 4 * MB * 1024; }  
 
 // MB: 16-row groups of X (M <= 16 * MB)
 template <int MB>
-__global__ void __launch_bounds__(256) hgemm_f16_fewrows_kernel(FewRowsArgs a) {
+__global__ void __launch_bounds__(256) hgemm_f16_fewrows_kernel(const half_t* p_X, const half_t* p_W, half_t* p_C, int p_M, int p_N,
+                                                                 int p_K, int p_ldc, int p_parts, int p_nblocks) {
+    // scalar parameters (preloaded into SGPRs with the wavefront), not the struct
+    const FewRowsArgs a{p_X, p_W, p_C, p_M, p_N, p_K, p_ldc, p_parts, p_nblocks};
     static_assert(MB == 1 || MB == 2, "X[16*MB, 1024] per wavefront must fit its registers");
     extern __shared__ __attribute__((aligned(1024))) unsigned char smem_raw[];
     typedef __attribute__((address_space(3))) unsigned char lds_byte_t;
@@ -242,7 +245,8 @@ static int launch_fewrows_variant(const FewRowsArgs& a) {
                                        hipFuncAttributeMaxDynamicSharedMemorySize, lds));
         attr_set.store(true);
     }
-    hipLaunchKernelGGL((hgemm_f16_fewrows_kernel<MB>), dim3((unsigned)a.parts), dim3(256), lds, stream(), a);
+    hipLaunchKernelGGL((hgemm_f16_fewrows_kernel<MB>), dim3((unsigned)a.parts), dim3(256), lds, stream(), a.X, a.W, a.C, a.M, a.N, a.K,
+                       a.ldc, a.parts, a.nblocks);
     TL_CHECK_LAUNCH("hgemm_f16_fewrows_kernel");
     return TL_OK;
 }
