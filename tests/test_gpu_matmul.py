@@ -853,6 +853,33 @@ def test_hgemm_256x128_agpr_kernel_integer_exact(dev, shape):
         dev.lib.tl_set_hgemm_k_rotation(-1, -1)
 
 
+def test_hgemm_agpr_kernels_drawn_whole_tile_shapes(dev):
+    """Twenty drawn whole-tile shapes per AGPR kernel (1 .. 6 rows of tiles, 1 .. 12 columns, 3 .. 40 K tiles), each under
+    a drawn tile band (the workgroup-to-tile map) and K rotation: small integers, exact."""
+    rng = np.random.default_rng(20241125)
+    names = dev.hgemm_variants()
+    try:
+        for name, bn, k_unit, k_min in (("a256x256x64w2x2", 256, 128, 256), ("a256x128x64w2x2", 128, 64, 192)):
+            dev.set_hgemm_variant(names.index(name))
+            for i in range(20):
+                M = 256 * int(rng.integers(1, 7))
+                N = bn * int(rng.integers(1, 13))
+                K = max(k_min, k_unit * int(rng.integers(1, 2560 // k_unit + 1)))
+                band = int(rng.choice([0, 1, 2, 3, 5, 8]))
+                rot = (int(rng.integers(0, 50)), int(rng.integers(0, 50))) if i % 2 else (-1, -1)
+                A = dev.from_numpy(synth.small_ints_f16(9700 + i, (M, K), -2, 2))
+                B = dev.from_numpy(synth.small_ints_f16(9800 + i, (N, K), -2, 2))
+                dev.lib.tl_set_hgemm_tile_band(band)
+                dev.lib.tl_set_hgemm_k_rotation(*rot)
+                C = dev.hgemm(A, B)
+                assert dev.hgemm_last_plan() == (name, 1), (name, M, N, K)
+                assert torch.equal(C.double(), A.double() @ B.double().T), (name, M, N, K, band, rot)
+    finally:
+        dev.set_hgemm_variant(0)
+        dev.lib.tl_set_hgemm_tile_band(0)
+        dev.lib.tl_set_hgemm_k_rotation(-1, -1)
+
+
 def test_hgemm_agpr_kernels_can_be_switched_off(dev):
     """tl_set_hgemm_agpr_kernels(-1) hands the shapes back to the ring kernels; both give the exact integer result."""
     A = dev.from_numpy(synth.small_ints_f16(9500, (2048, 512), -2, 2))
