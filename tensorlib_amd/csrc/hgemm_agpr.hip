@@ -29,6 +29,11 @@
 // travelling through registers (two K tiles in flight per wavefront, ds_write_b128 into the same ring) was built too,
 // for either operand or both: 433 us on the first shape.  A ds_write_b128 occupies the LDS pipeline five times as long
 // as a fragment read of the same size, which costs more than the deeper prefetch returns.
+// What is left between the measured 0.77-0.81 matrix-core occupancy and 1: per K tile a workgroup writes 64 KB into LDS
+// (DMA) and reads 128 KB of fragments out of it, 192 KB against 2048 MFMA cycles, i.e. 94 of the 128 bytes per clock the LDS
+// moves; a 2x2 arrangement of 128x128 wavefront tiles is the one with the fewest LDS bytes per flop that 512 registers per
+// lane allow.  Measured and ruled out: L2 miss latency (W resident in the memory-side cache, a prefetching fifth
+// wavefront), the request spacing and barrier position, the four wavefronts issuing requests in the same slots.
 #include <atomic>
 #include <type_traits>
 
