@@ -63,6 +63,9 @@ def parse_args():
                          "1 inside the GEMM launch")
     ap.add_argument("--hgemm-variant", default="",
                     help="--workload hgemm: force one kernel variant by name (tl_hgemm_variant_name), default dispatch")
+    ap.add_argument("--vendor-reference", action="store_true",
+                    help="--workload hgemm: time torch.matmul (hipBLASLt) on the same operands next to the library, "
+                         "alternating, and report both per shape in extra.hgemm_prefill")
     ap.add_argument("--no-extra", action="store_true", help="skip the HGEMM / per-shape / model extras")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--copy-calibration", action="store_true",
@@ -196,7 +199,10 @@ def mfma_sustained(dev):
     return out
 
 
-def hgemm_table(dev, randn, torch, synth, sustained_tf, shapes=None):
+def hgemm_table(dev, randn, torch, synth, sustained_tf, shapes=None, vendor=False):
+    """Per-shape times of tl_matmul2d_f16 with W streamed from HBM.  vendor: also time torch.matmul (hipBLASLt / rocBLAS
+    behind it) on the same operands, alternating with the library in three rounds, minimum kept for both: a reference
+    point on the same box, not a product path."""
     hg = {}
     for (M, N, K) in (shapes or HGEMM_SHAPES):
         A = randn((M, K), 1.0)
@@ -214,6 +220,18 @@ def hgemm_table(dev, randn, torch, synth, sustained_tf, shapes=None):
             one()
         reps = 40
         _, ev1 = time_region(one, reps, torch)
+        vendor_us = None
+        if vendor:
+            def other():
+                it[0] += 1
+                torch.matmul(A, Bs[it[0] % nb].T, out=C)
+            for _ in range(5):
+                other()
+            vendor_ev = []
+            for _ in range(3):
+                vendor_ev.append(time_region(other, reps, torch)[1])
+                ev1 = min(ev1, time_region(one, reps, torch)[1])
+            vendor_us = min(vendor_ev) / reps * 1e6
         del Bs
         us = ev1 / reps * 1e6
         tf = synth.gemm_flops(M, N, K) / us / 1e6
@@ -225,6 +243,9 @@ def hgemm_table(dev, randn, torch, synth, sustained_tf, shapes=None):
                               "bound": "mfma" if bound_tf >= MFMA_FP16_PEAK_TFLOPS else "hbm",
                               "frac_of_bound": round(tf / bound_tf, 4),
                               "frac_of_sustained_mfma": round(tf / sustained_tf, 4)}
+        if vendor_us is not None:
+            hg[f"{M}x{N}x{K}"]["torch_matmul_us"] = round(vendor_us, 1)
+            hg[f"{M}x{N}x{K}"]["us_over_torch_matmul_us"] = round(us / vendor_us, 3)
     return hg
 
 
@@ -472,7 +493,8 @@ def main():
                          "sustained_mfma_tflops": sustained},
         }
         if not args.no_extra:
-            out["extra"] = {"hgemm_prefill": hgemm_table(dev, randn, torch, synth, max(sustained["changing_operands"], sustained["changing_operands_16x16x32"]), shapes)}
+            out["extra"] = {"hgemm_prefill": hgemm_table(dev, randn, torch, synth, max(sustained["changing_operands"], sustained["changing_operands_16x16x32"]), shapes,
+                                                         vendor=args.vendor_reference)}
         if not args.no_cpu:
             out["cpu_baseline"] = cpu_baseline_hgemm()
         print(json.dumps(out))
